@@ -1,0 +1,156 @@
+/*
+ * wkf_tensor.h -- level 1 of the C ABI: the lazy Tensor API of the reference
+ * crate (`Tensor<const R, D>`, re-exported by src/lib.rs:1-11) behind opaque C
+ * handles.  A Rust `Tensor<R, D>` facade binds these one-to-one (INTEGRATION.md
+ * shows the `extern "C"` block); ranks and dtypes are checked at run time where
+ * the Rust types check them at compile time.
+ *
+ * Every op only records a node (src/tensor.rs:179-284); nothing touches the GPU
+ * until wkf_tensor_materialize / wkf_tensor_as_slice.  Where the reference
+ * panics (shape mismatch, bad axis ...) these return WKF_ERR_INVALID_ARG and
+ * leave the message in wkf_last_error().
+ *
+ * Paths in comments are relative to the reference checkout.
+ */
+#ifndef WKF_TENSOR_H
+#define WKF_TENSOR_H
+
+#include "wkf_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct wkf_tensor wkf_tensor;
+typedef struct wkf_slice wkf_slice;
+
+/* DataTypeEnum, src/tensor.rs:69-88 */
+enum { WKF_F32 = 0, WKF_F16 = 1 };
+
+/* Element-wise functions.  tensor-with-literal: src/element_wise.rs:197-675. */
+enum {
+  WKF_OP_ADD_CONST = 0, /* t + c, c + t   :197-271 */
+  WKF_OP_SUB_CONST = 1, /* t - c          :445-458 */
+  WKF_OP_CONST_SUB = 2, /* c - t          :485-498 */
+  WKF_OP_MUL_CONST = 3, /* t * c, c * t   :525-571 */
+  WKF_OP_DIV_CONST = 4, /* t / c          :598-611 */
+  WKF_OP_CONST_DIV = 5, /* c / t          :638-651 */
+  /* unary: src/element_wise.rs:678-1380 */
+  WKF_OP_EXP = 16, WKF_OP_EXP2, WKF_OP_LOG, WKF_OP_LOG2, WKF_OP_SQR, WKF_OP_SQRT, WKF_OP_SIN, WKF_OP_COS,
+  WKF_OP_TAN, WKF_OP_ASIN, WKF_OP_ACOS, WKF_OP_ATAN, WKF_OP_SINH, WKF_OP_COSH, WKF_OP_TANH, WKF_OP_ASINH,
+  WKF_OP_ACOSH, WKF_OP_ATANH, WKF_OP_ABS, WKF_OP_NEG,
+  /* pair-wise: src/pair_wise.rs:205-528 */
+  WKF_OP_ADD = 64, WKF_OP_SUB, WKF_OP_MUL, WKF_OP_DIV, WKF_OP_POW
+};
+
+/* src/reduce.rs:433-815 */
+enum { WKF_REDUCE_SUM = 0, WKF_REDUCE_MAX = 1, WKF_REDUCE_MIN = 2, WKF_REDUCE_PRODUCT = 3 };
+
+/* Which fusion rules the executor applies on this device.
+ * WKF_FUSION_REFERENCE: exactly src/compute_graph/resolve.rs:49-196 (element-wise
+ *   chains fuse into one kernel, into the two operands and the result of ONE
+ *   pair-wise op, and before/after a reduce; nothing else fuses; a node used
+ *   twice is computed twice).
+ * WKF_FUSION_TREE (default): additionally whole pair-wise trees, and the copies
+ *   of resize / slice_assign, fuse with the element-wise work around them, and a
+ *   node used twice is computed once.  Every op is still rounded on its own, so
+ *   results are identical to the reference rules. */
+enum { WKF_FUSION_REFERENCE = 0, WKF_FUSION_TREE = 1 };
+int wkf_device_set_fusion(wkf_device* dev, int mode);
+int wkf_device_get_fusion(wkf_device* dev);
+
+/* Accuracy of exp / sin / cos and the other transcendental ops (no reference
+ * counterpart: the reference leaves them to the WGSL driver, which only bounds
+ * them, e.g. exp to 3 + 2|x| ulp).
+ * Default (0): an op whose value feeds further arithmetic of the same kernel is
+ *   evaluated in f64 and rounded once (it equals the correctly rounded f32 value,
+ *   so later ops cannot amplify an error); the last op before a store uses the
+ *   f32 library (<= 1-2 ulp); values that only feed a reduction use the f32 library.
+ * exact != 0: every transcendental op is evaluated in f64 and rounded once. */
+int wkf_device_set_exact_math(wkf_device* dev, int exact);
+
+/* Tensor::new, src/tensor.rs:518-531 (+ IntoTensor :441-515): uploads `data`
+ * (row-major, numel * sizeof(dtype) bytes) into a new leaf tensor. */
+int wkf_tensor_new(wkf_device* dev, int dtype, int rank, const size_t* shape, const void* data, wkf_tensor** out);
+/* Clone of a handle (Tensor: Clone, src/tensor.rs:435-442): same node. */
+int wkf_tensor_clone(const wkf_tensor* t, wkf_tensor** out);
+void wkf_tensor_free(wkf_tensor* t);
+int wkf_tensor_rank(const wkf_tensor* t);                 /* Tensor::rank, src/tensor.rs:634-636 */
+int wkf_tensor_shape(const wkf_tensor* t, size_t* out);   /* Tensor::shape, :630-632 */
+int wkf_tensor_dtype(const wkf_tensor* t);                /* Tensor::datatype, :638-640 */
+
+/* t (op) c with an f32 literal; op is one of WKF_OP_*_CONST / WKF_OP_CONST_*. */
+int wkf_tensor_scalar_op(const wkf_tensor* t, int op, float c, wkf_tensor** out);
+/* exp ... neg */
+int wkf_tensor_unary_op(const wkf_tensor* t, int op, wkf_tensor** out);
+/* Tensor::cast, src/element_wise.rs:1408-1471 (T -> T records no node). */
+int wkf_tensor_cast(const wkf_tensor* t, int dtype, wkf_tensor** out);
+/* add sub mul div pow; shapes and dtypes must be equal (src/pair_wise.rs:92). */
+int wkf_tensor_binary_op(const wkf_tensor* a, const wkf_tensor* b, int op, wkf_tensor** out);
+/* Sum::sum / Max::max / Min::min / Product::product over `axis`; rank drops by one. */
+int wkf_tensor_reduce(const wkf_tensor* t, int reduce_op, size_t axis, wkf_tensor** out);
+/* Tensor::mat_mul, src/matmul.rs:25-29: rank 2, same dtype, [M,K] x [K,N]. */
+int wkf_tensor_mat_mul(const wkf_tensor* a, const wkf_tensor* b, wkf_tensor** out);
+
+/* Zero-copy views, src/map_layout.rs:42-98. */
+int wkf_tensor_slice(const wkf_tensor* t, const size_t* starts, const size_t* ends, wkf_tensor** out);
+int wkf_tensor_transpose(const wkf_tensor* t, size_t first_axis, size_t second_axis, wkf_tensor** out);
+int wkf_tensor_broadcast(const wkf_tensor* t, int out_rank, const size_t* out_shape, wkf_tensor** out);
+/* src/composite/narrow.rs:3-16 */
+int wkf_tensor_narrow(const wkf_tensor* t, size_t axis, size_t start, size_t length, wkf_tensor** out);
+
+/* Copies, src/resize.rs:121-145, src/composite/unsqueeze.rs:3-53. */
+int wkf_tensor_resize(const wkf_tensor* t, const size_t* new_shape, wkf_tensor** out);
+int wkf_tensor_reshape(const wkf_tensor* t, int new_rank, const size_t* new_shape, wkf_tensor** out);
+int wkf_tensor_unsqueeze(const wkf_tensor* t, size_t axis, wkf_tensor** out);
+/* src/slice_assign.rs:76-80 */
+int wkf_tensor_slice_assign(const wkf_tensor* t, const size_t* starts, const size_t* ends, const wkf_tensor* value,
+                            wkf_tensor** out);
+/* Tensor::cat, src/composite/cat.rs:3-41 */
+int wkf_tensor_cat(const wkf_tensor* const* tensors, int count, size_t dim, wkf_tensor** out);
+
+/* Composites, src/composite/{silu,rms_norm,rope,softmax,arange}.rs */
+int wkf_tensor_silu(const wkf_tensor* t, wkf_tensor** out);
+/* `layer_norm` of the reference is RMSNorm: (x / sqrt(mean(x^2) + eps)) * weight, computed in f32. */
+int wkf_tensor_layer_norm(const wkf_tensor* t, const wkf_tensor* weight, float eps, wkf_tensor** out);
+/* rope: t [heads, seq, dim]; cos/sin [max_seq, dim/2] (duplicated on the last dim) or [max_seq, dim]. */
+int wkf_tensor_rope(const wkf_tensor* t, const wkf_tensor* cos, const wkf_tensor* sin, wkf_tensor** out);
+/* rank-1 softmax exactly as src/composite/softmax.rs:4-10 (no max subtraction). */
+int wkf_tensor_softmax(const wkf_tensor* t, wkf_tensor** out);
+/* Max-subtracted softmax over the last dim of any rank, built from the same
+ * primitives (max, sub, exp, sum, div); not in the reference. */
+int wkf_tensor_softmax_last_dim(const wkf_tensor* t, wkf_tensor** out);
+/* arange / arange_step, src/composite/arange.rs:4-23 (host loop + upload). */
+int wkf_tensor_arange(wkf_device* dev, int dtype, float start, float end, float step, wkf_tensor** out);
+
+/* LazyTensorData::materialize, src/tensor.rs:286-288: run the graph under `t`.
+ * The result stays on the device; kernels are timed with a hipEvent pair each. */
+int wkf_tensor_materialize(wkf_tensor* t);
+/* Tensor::all_timing_information, src/tensor.rs:556-558: number of kernels the
+ * last materialize launched, and for kernel `i` its elapsed time, kind and
+ * cache signature. */
+int wkf_tensor_kernel_count(const wkf_tensor* t);
+int wkf_tensor_kernel_info(const wkf_tensor* t, int i, uint64_t* elapsed_ns, char* kind, size_t kind_cap,
+                           char* signature, size_t signature_cap, char* detail, size_t detail_cap);
+/* The generated HIP source of a kernel signature seen by this process (for inspection and tests). */
+int wkf_kernel_source(const char* signature, char* out, size_t cap, size_t* needed);
+
+/* Tensor::as_slice, src/tensor.rs:533-554: materialise, download the WHOLE
+ * buffer, and keep the layout so that strided views are decoded on the host
+ * (TensorSlice, src/tensor.rs:669-855). */
+int wkf_tensor_as_slice(wkf_tensor* t, wkf_slice** out);
+void wkf_slice_free(wkf_slice* s);
+int wkf_slice_rank(const wkf_slice* s);
+int wkf_slice_dtype(const wkf_slice* s);
+/* layout: offset, shape[rank], strides[rank], all in elements */
+int wkf_slice_layout(const wkf_slice* s, size_t* offset, size_t* shape, size_t* strides);
+/* Pointer to element 0 of the downloaded buffer and its size in bytes. */
+const void* wkf_slice_data(const wkf_slice* s, size_t* bytes);
+/* TensorSlice::get, src/tensor.rs:827-846: 0 and the element widened to f32, or
+ * WKF_ERR_INVALID_ARG when an index is out of range. */
+int wkf_slice_get(const wkf_slice* s, const size_t* index, float* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,539 @@
+#include "codegen.h"
+
+#include <cstring>
+#include <sstream>
+
+namespace wkf {
+namespace {
+
+const char* ctype(DType d) { return d == DType::F32 ? "float" : "_Float16"; }
+
+std::string vtype(DType d, int v) {
+  if (v == 1) return ctype(d);
+  return std::string(d == DType::F32 ? "wkf_f32x" : "wkf_f16x") + std::to_string(v);
+}
+
+// Shared by every generated translation unit.
+const char* const kPrelude =
+#include "kernels/prelude.hip.inc"
+    ;
+
+// exp / sin / cos with f64 Taylor cores; appended only to kernels that use them.
+const char* const kMath =
+#include "kernels/math.hip.inc"
+    ;
+
+// True when instruction i of p is evaluated with an f64 core under `policy`.
+bool exact_op(const Program& p, size_t i, MathPolicy policy) {
+  if (policy == MathPolicy::Exact) return true;
+  if (policy == MathPolicy::Folded) return false;
+  for (size_t j = i + 1; j < p.ins.size(); j++)
+    if (p.ins[j].a == int(i) || p.ins[j].b == int(i)) return true;  // interior: something reads it
+  return false;
+}
+
+bool has_core(Op o) { return o == Op::Exp || o == Op::Sin || o == Op::Cos; }
+
+// Needs the f64 cores of kernels/math.hip.inc.
+bool uses_math(const Program& p, MathPolicy policy) {
+  for (size_t i = 0; i < p.ins.size(); i++)
+    if (has_core(p.ins[i].op) && exact_op(p, i, policy)) return true;
+  return false;
+}
+
+// Uses the branch-free sin / cos core, i.e. needs the `far` flag and a far variant.
+bool uses_trig(const Program& p, MathPolicy policy) {
+  for (size_t i = 0; i < p.ins.size(); i++)
+    if ((p.ins[i].op == Op::Sin || p.ins[i].op == Op::Cos) && exact_op(p, i, policy)) return true;
+  return false;
+}
+
+const char* lib_fn(Op o) {
+  switch (o) {
+    case Op::Exp: return "exp";
+    case Op::Exp2: return "exp2";
+    case Op::Log: return "log";
+    case Op::Log2: return "log2";
+    case Op::Sqrt: return "sqrt";
+    case Op::Sin: return "sin";
+    case Op::Cos: return "cos";
+    case Op::Tan: return "tan";
+    case Op::Asin: return "asin";
+    case Op::Acos: return "acos";
+    case Op::Atan: return "atan";
+    case Op::Sinh: return "sinh";
+    case Op::Cosh: return "cosh";
+    case Op::Tanh: return "tanh";
+    case Op::Asinh: return "asinh";
+    case Op::Acosh: return "acosh";
+    case Op::Atanh: return "atanh";
+    default: return nullptr;
+  }
+}
+
+// f32 -> f32 call text of a unary math op on the f32 expression `a`.
+std::string math_call(Op o, const std::string& a, bool exact, bool far_variant) {
+  const std::string f = lib_fn(o);
+  if (o == Op::Sqrt || !exact) return f + "f(" + a + ")";  // sqrtf is correctly rounded already
+  if (o == Op::Exp) return "wkf_exp(" + a + ")";
+  if (o == Op::Sin || o == Op::Cos) return "wkf_" + f + (far_variant ? "_far(" + a + ")" : "(" + a + ", far)");
+  return "(float)" + f + "((double)(" + a + "))";  // the library's f64 routine, rounded once
+}
+
+// Emits `static __device__ RT name(T0 x0, ..., const float* c[, bool& far])`: one
+// statement per fused op, each result held in a variable of the op's own dtype so
+// that it is rounded before the next op reads it (src/kernel.rs:540-553 gives
+// every fused function a typed signature for the same effect).
+// A program with sin / cos gets two functions: `name`, whose branch-free trig sets
+// `far` when an argument is outside its exact range, and `name_far`, which goes
+// through the library's f64 sin / cos and is called to redo the work when `far`.
+void emit_program_variant(std::ostringstream& o, const Program& p, const std::string& name,
+                          const std::vector<DType>& operand_types, MathPolicy policy, bool far_variant) {
+  const bool trig = uses_trig(p, policy);
+  o << "static __device__ " << (far_variant ? "__attribute__((noinline)) " : "__forceinline__ ") << ctype(p.result_dtype())
+    << " " << name << (far_variant ? "_far" : "") << "(";
+  for (size_t i = 0; i < operand_types.size(); i++) o << ctype(operand_types[i]) << " x" << i << ", ";
+  o << "const float* c" << (trig && !far_variant ? ", bool& far" : "") << ") {\n";
+  for (size_t i = 0; i < p.ins.size(); i++) {
+    const Instr& in = p.ins[i];
+    const bool h = in.dtype == DType::F16;
+    const char* t = ctype(in.dtype);
+    std::string a = "v" + std::to_string(in.a), b = "v" + std::to_string(in.b);
+    std::string k = h ? "(_Float16)c[" + std::to_string(in.cslot) + "]" : "c[" + std::to_string(in.cslot) + "]";
+    o << "  const " << t << " v" << i << " = ";
+    switch (in.op) {
+      case Op::Load: o << "x" << in.operand; break;
+      case Op::AddC: o << a << " + " << k; break;
+      case Op::SubC: o << a << " - " << k; break;
+      case Op::RSubC: o << k << " - " << a; break;
+      case Op::MulC: o << a << " * " << k; break;
+      case Op::DivC: o << a << " / " << k; break;
+      case Op::RDivC: o << k << " / " << a; break;
+      case Op::Sqr: o << a << " * " << a; break;
+      case Op::Neg: o << "-" << a; break;
+      case Op::Abs:
+        if (h) o << "(_Float16)__builtin_fabsf((float)" << a << ")";
+        else o << "__builtin_fabsf(" << a << ")";
+        break;
+      case Op::Cast: o << "(" << t << ")" << a; break;
+      case Op::Add: o << a << " + " << b; break;
+      case Op::Sub: o << a << " - " << b; break;
+      case Op::Mul: o << a << " * " << b; break;
+      case Op::Div: o << a << " / " << b; break;
+      case Op::Pow: {
+        const bool exact = exact_op(p, i, policy);
+        std::string call = exact ? "(float)pow((double)" + a + ", (double)" + b + ")"
+                                 : (h ? "powf((float)" + a + ", (float)" + b + ")" : "powf(" + a + ", " + b + ")");
+        o << (h ? "(_Float16)" : "") << call;
+        break;
+      }
+      default: {
+        std::string call = math_call(in.op, h ? "(float)" + a : a, exact_op(p, i, policy), far_variant);
+        o << (h ? "(_Float16)" : "") << call;
+      }
+    }
+    o << ";\n";
+  }
+  o << "  return v" << p.result << ";\n}\n";
+}
+
+void emit_program(std::ostringstream& o, const Program& p, const std::string& name,
+                  const std::vector<DType>& operand_types, MathPolicy policy) {
+  emit_program_variant(o, p, name, operand_types, policy, false);
+  if (uses_trig(p, policy)) emit_program_variant(o, p, name, operand_types, policy, true);
+}
+
+void put32(std::vector<unsigned char>& b, uint32_t v) {
+  unsigned char t[4];
+  memcpy(t, &v, 4);
+  b.insert(b.end(), t, t + 4);
+}
+void putf(std::vector<unsigned char>& b, float v) {
+  unsigned char t[4];
+  memcpy(t, &v, 4);
+  b.insert(b.end(), t, t + 4);
+}
+void putp(std::vector<unsigned char>& b, const void* v) {
+  unsigned char t[8];
+  memcpy(t, &v, 8);
+  b.insert(b.end(), t, t + 8);
+}
+void pad8(std::vector<unsigned char>& b) {
+  while (b.size() % 8) b.push_back(0);
+}
+
+}  // namespace
+
+// ===========================================================================
+// map kernels
+// ===========================================================================
+
+std::string map_signature(const MapSpec& s) {
+  std::ostringstream o;
+  o << "map|gfx950|r" << s.rank << "|v" << s.vec << "|u" << s.unroll << (s.nontemporal ? "|nt" : "|ca") << "|in:";
+  for (const auto& i : s.in) o << dtype_name(i.dtype) << (i.linear ? 'L' : 'S') << i.inner_stride << ',';
+  o << "|out:" << dtype_name(s.out.dtype) << (s.out.linear ? 'L' : 'S') << s.out.inner_stride;
+  o << "|m" << int(s.math) << "|" << s.prog.signature();
+  return o.str();
+}
+
+std::string map_source(const MapSpec& s) {
+  const int N = int(s.in.size()) + 1;  // operands incl. out
+  const int R = s.rank, V = s.vec, U = s.unroll;
+  const int NC = s.prog.consts.empty() ? 1 : int(s.prog.consts.size());
+  std::ostringstream o;
+  o << kPrelude;
+  if (uses_math(s.prog, s.math)) o << kMath;
+  o << "struct Args { void* p[" << N << "]; u32 nwork; u32 shape[" << R << "]; u32 off[" << N << "]; u32 stride[" << N
+    << "][" << R << "]; float c[" << NC << "]; };\n";
+  std::vector<DType> types;
+  for (const auto& i : s.in) types.push_back(i.dtype);
+  emit_program(o, s.prog, "wkf_expr", types, s.math);
+
+  bool need_unravel = false;
+  for (const auto& i : s.in) need_unravel |= !i.linear;
+  need_unravel |= !s.out.linear;
+
+  auto operand = [&](int k) -> const MapOperandSpec& { return k < N - 1 ? s.in[k] : s.out; };
+  auto index_expr = [&](int k, int j) {
+    const MapOperandSpec& op = operand(k);
+    std::ostringstream e;
+    std::string w = "w" + std::to_string(j);
+    if (op.linear) {
+      e << "a.off[" << k << "] + " << w << " * " << V << "u";
+      return e.str();
+    }
+    e << "a.off[" << k << "]";
+    for (int d = 0; d < R - 1; d++) e << " + i" << d << "_" << j << " * a.stride[" << k << "][" << d << "]";
+    if (op.inner_stride == 1) e << " + i" << R - 1 << "_" << j << " * " << V << "u";
+    else if (op.inner_stride < 0) e << " + i" << R - 1 << "_" << j << " * a.stride[" << k << "][" << R - 1 << "]";
+    return e.str();
+  };
+  // A vector operand whose inner stride is 0 is one scalar broadcast to every lane of the work item.
+  auto is_vec_load = [&](int k) { return V > 1 && (operand(k).linear || operand(k).inner_stride == 1); };
+
+  auto emit_index = [&](int j, const char* ind) {
+    o << ind << "const u32 w" << j << " = w_first + " << j * kMapBlock << "u;\n";
+    if (need_unravel) {
+      o << ind << "u32 rem" << j << " = w" << j << ";\n";
+      for (int d = R - 1; d > 0; d--) {
+        o << ind << "const u32 i" << d << "_" << j << " = rem" << j << " % a.shape[" << d << "]; rem" << j
+          << " /= a.shape[" << d << "];\n";
+      }
+      o << ind << "const u32 i0_" << j << " = rem" << j << ";\n";
+    }
+  };
+  auto emit_loads = [&](int j, const char* ind) {
+    for (int k = 0; k < N - 1; k++) {
+      const MapOperandSpec& op = s.in[k];
+      std::string ptr = std::string("((const ") + ctype(op.dtype) + "*)a.p[" + std::to_string(k) + "])";
+      if (is_vec_load(k)) {
+        std::string vt = vtype(op.dtype, V);
+        o << ind << "const " << vt << " r" << k << "_" << j << " = ";
+        if (s.nontemporal && op.linear)
+          o << "__builtin_nontemporal_load((const " << vt << "*)(" << ptr << " + (" << index_expr(k, j) << ")));\n";
+        else
+          o << "*(const " << vt << "*)(" << ptr << " + (" << index_expr(k, j) << "));\n";
+      } else {
+        o << ind << "const " << ctype(op.dtype) << " r" << k << "_" << j << " = " << ptr << "[" << index_expr(k, j)
+          << "];\n";
+      }
+    }
+  };
+  const bool trig = uses_trig(s.prog, s.math);
+  const std::string ot = vtype(s.out.dtype, V);
+  const std::string optr = std::string("((") + ctype(s.out.dtype) + "*)a.p[" + std::to_string(N - 1) + "])";
+  auto emit_compute = [&](int j, const char* ind, bool far_variant) {
+    for (int e = 0; e < V; e++) {
+      o << ind << "o" << j;
+      if (V > 1) o << "[" << e << "]";
+      o << " = wkf_expr" << (far_variant ? "_far" : "") << "(";
+      for (int k = 0; k < N - 1; k++) {
+        o << "r" << k << "_" << j;
+        if (is_vec_load(k)) o << "[" << e << "]";
+        o << ", ";
+      }
+      o << "a.c" << (trig && !far_variant ? ", far" : "") << ");\n";
+    }
+  };
+  auto emit_store = [&](int j, const char* ind) {
+    if (V > 1) {
+      if (s.nontemporal && s.out.linear)
+        o << ind << "__builtin_nontemporal_store(o" << j << ", (" << ot << "*)(" << optr << " + (" << index_expr(N - 1, j)
+          << ")));\n";
+      else
+        o << ind << "*(" << ot << "*)(" << optr << " + (" << index_expr(N - 1, j) << ")) = o" << j << ";\n";
+    } else {
+      o << ind << optr << "[" << index_expr(N - 1, j) << "] = o" << j << ";\n";
+    }
+  };
+  // loads -> fused expression on every element -> (rarely) redo through the far variant -> stores
+  auto emit_batch = [&](int j0, int j1, const std::string& ind) {
+    for (int j = j0; j < j1; j++) emit_loads(j, ind.c_str());
+    for (int j = j0; j < j1; j++) o << ind << ot << " o" << j << ";\n";
+    if (trig) o << ind << "bool far = false;\n";
+    for (int j = j0; j < j1; j++) emit_compute(j, ind.c_str(), false);
+    if (trig) {
+      o << ind << "if (__builtin_expect(far, 0)) {\n";
+      for (int j = j0; j < j1; j++) emit_compute(j, (ind + "  ").c_str(), true);
+      o << ind << "}\n";
+    }
+    for (int j = j0; j < j1; j++) emit_store(j, ind.c_str());
+  };
+
+  o << "extern \"C\" __global__ void __launch_bounds__(" << kMapBlock << ") wkf_kernel(const Args a) {\n";
+  o << "  const u32 w_block = blockIdx.x * " << kMapBlock * U << "u;\n";
+  o << "  const u32 w_first = w_block + threadIdx.x;\n";
+  o << "  if (w_block + " << kMapBlock * U << "u <= a.nwork) {\n";
+  // Full block: every load is issued before the first use so that U independent
+  // 16-byte requests per operand are in flight per lane.
+  for (int j = 0; j < U; j++) emit_index(j, "    ");
+  emit_batch(0, U, "    ");
+  o << "  } else {\n";
+  for (int j = 0; j < U; j++) {
+    o << "    {\n";
+    emit_index(j, "      ");
+    o << "      if (w" << j << " < a.nwork) {\n";
+    emit_batch(j, j + 1, "        ");
+    o << "      }\n    }\n";
+  }
+  o << "  }\n}\n";
+  return o.str();
+}
+
+std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a) {
+  const size_t N = s.in.size() + 1;
+  const size_t R = size_t(s.rank);
+  if (a.ptrs.size() != N || a.shape.size() != R || a.offsets.size() != N || a.strides.size() != N)
+    throw Error(WKF_ERR_INVALID_ARG, "map_pack_args: argument arity does not match the kernel");
+  std::vector<unsigned char> b;
+  for (void* p : a.ptrs) putp(b, p);
+  put32(b, a.nwork);
+  for (uint32_t v : a.shape) put32(b, v);
+  for (uint32_t v : a.offsets) put32(b, v);
+  for (const auto& st : a.strides) {
+    if (st.size() != R) throw Error(WKF_ERR_INVALID_ARG, "map_pack_args: stride rank mismatch");
+    for (uint32_t v : st) put32(b, v);
+  }
+  size_t nc = s.prog.consts.empty() ? 1 : s.prog.consts.size();
+  for (size_t i = 0; i < nc; i++) putf(b, i < a.consts.size() ? a.consts[i] : 0.f);
+  pad8(b);
+  return b;
+}
+
+// ===========================================================================
+// reduce kernels
+// ===========================================================================
+
+namespace {
+const char* fold_macro(ReduceOp r) {
+  // The reference always calls the combine as f(new_value, merged), src/reduce.rs:183,204,254.
+  switch (r) {
+    case ReduceOp::Sum: return "#define WKF_FOLD(v, acc) ((v) + (acc))\n#define WKF_SEED 0.0f\n";
+    case ReduceOp::Max: return "#define WKF_FOLD(v, acc) fmaxf((v), (acc))\n#define WKF_SEED (-3.40282e+38f)\n";
+    case ReduceOp::Min: return "#define WKF_FOLD(v, acc) fminf((v), (acc))\n#define WKF_SEED (3.40282e+38f)\n";
+    case ReduceOp::Product: return "#define WKF_FOLD(v, acc) ((v) * (acc))\n#define WKF_SEED 1.0f\n";
+  }
+  return "";
+}
+const char* const kReduceHelpers =
+#include "kernels/reduce_helpers.hip.inc"
+    ;
+}  // namespace
+
+std::string reduce_signature(const ReduceSpec& s) {
+  std::ostringstream o;
+  o << (s.shape == ReduceShape::Row ? "red_row" : "red_col") << "|gfx950|" << reduce_name(s.rop) << "|or" << s.outer_rank
+    << "|v" << s.vec << "|t" << s.threads_per_row << "|b" << s.block << "|u" << s.unroll << "|w" << s.waves << "|in:";
+  for (const auto& i : s.in) o << dtype_name(i.dtype) << 'a' << i.axis_stride << ',';
+  o << "|out:" << dtype_name(s.out_dtype) << "|m" << int(s.math_pre) << int(s.math_post) << "|pre:" << s.pre.signature()
+    << "|post:" << s.post.signature();
+  return o.str();
+}
+
+std::string reduce_source(const ReduceSpec& s) {
+  const int N = int(s.in.size());
+  const int Ro = s.outer_rank;
+  const int NCpre = int(s.pre.consts.size());
+  const int NC = std::max(1, NCpre + int(s.post.consts.size()));
+  const DType pre_dt = s.pre.result_dtype();
+  std::ostringstream o;
+  o << kPrelude;
+  if (uses_math(s.pre, s.math_pre) || uses_math(s.post, s.math_post)) o << kMath;
+  o << fold_macro(s.rop);
+  o << kReduceHelpers;
+  o << "struct Args { void* p[" << N + 1 << "]; u32 nrows; u32 n; u32 nvec; u32 oshape[" << std::max(1, Ro)
+    << "]; u32 off[" << N + 1 << "]; u32 ostride[" << N + 1 << "][" << std::max(1, Ro) << "]; u32 astride["
+    << std::max(1, N) << "]; float c[" << NC << "]; };\n";
+  std::vector<DType> types;
+  for (const auto& i : s.in) types.push_back(i.dtype);
+  emit_program(o, s.pre, "wkf_pre", types, s.math_pre);
+  emit_program(o, s.post, "wkf_post", {pre_dt}, s.math_post);
+
+  auto unravel = [&](const char* row, const char* ind) {
+    // i_d = index along outer dim d of output element `row`
+    if (Ro == 0) return;
+    o << ind << "u32 rem = " << row << ";\n";
+    for (int d = Ro - 1; d > 0; d--)
+      o << ind << "const u32 i" << d << " = rem % a.oshape[" << d << "]; rem /= a.oshape[" << d << "];\n";
+    o << ind << "const u32 i0 = rem;\n";
+  };
+  auto base_expr = [&](int k) {
+    std::ostringstream e;
+    e << "a.off[" << k << "]";
+    for (int d = 0; d < Ro; d++) e << " + i" << d << " * a.ostride[" << k << "][" << d << "]";
+    return e.str();
+  };
+  auto ptr = [&](int k) { return std::string("((const ") + ctype(s.in[k].dtype) + "*)a.p[" + std::to_string(k) + "])"; };
+  // the folded value is rounded to the tensor dtype, then `post` runs in that dtype
+  // A post chain with sin / cos runs once per output, so it simply takes the far variant.
+  std::string store_value = std::string(uses_trig(s.post, s.math_post) ? "wkf_post_far((" : "wkf_post((") + ctype(pre_dt) + ")acc, a.c + " +
+                            std::to_string(NCpre) + ")";
+  std::string out_ptr = std::string("((") + ctype(s.out_dtype) + "*)a.p[" + std::to_string(N) + "])";
+
+  if (s.shape == ReduceShape::Row) {
+    const int T = s.threads_per_row, V = s.vec, U = s.unroll, B = s.block;
+    const int RPB = B / T;
+    o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") wkf_kernel(const Args a) {\n";
+    if (T > 64) o << "  __shared__ float wkf_partial[" << B / 64 << "];\n";
+    o << "  const u32 t = threadIdx.x % " << T << "u;\n";
+    o << "  const u32 row_raw = blockIdx.x * " << RPB << "u + threadIdx.x / " << T << "u;\n";
+    o << "  const bool live = row_raw < a.nrows;\n";
+    o << "  const u32 row = live ? row_raw : 0u;\n";  // dead lanes redo row 0 so every lane reaches the barriers
+    unravel("row", "  ");
+    for (int k = 0; k < N; k++) {
+      o << "  const " << ctype(s.in[k].dtype) << "* q" << k << " = " << ptr(k) << " + (" << base_expr(k) << ");\n";
+      if (s.in[k].axis_stride == 0) o << "  const " << ctype(s.in[k].dtype) << " s" << k << " = q" << k << "[0];\n";
+    }
+    o << "  float acc = WKF_SEED;\n";
+    auto emit_loads = [&](int j, const char* ind) {
+      for (int k = 0; k < N; k++) {
+        if (s.in[k].axis_stride == 0) continue;
+        std::string vt = vtype(s.in[k].dtype, V);
+        o << ind << "const " << vt << " r" << k << "_" << j << " = ";
+        if (V > 1) o << "__builtin_nontemporal_load((const " << vt << "*)(q" << k << " + (k + " << j * T << "u) * " << V << "u));\n";
+        else o << "q" << k << "[k + " << j * T << "u];\n";
+      }
+    };
+    const bool trig = uses_trig(s.pre, s.math_pre);
+    auto emit_values = [&](int j, const char* ind, bool far_variant) {
+      for (int e = 0; e < V; e++) {
+        o << ind << "t" << j << "_" << e << " = wkf_pre" << (far_variant ? "_far" : "") << "(";
+        for (int k = 0; k < N; k++) {
+          if (s.in[k].axis_stride == 0) o << "s" << k;
+          else {
+            o << "r" << k << "_" << j;
+            if (V > 1) o << "[" << e << "]";
+          }
+          o << ", ";
+        }
+        o << "a.c" << (trig && !far_variant ? ", far" : "") << ");\n";
+      }
+    };
+    // loads -> pre on every element -> (rarely) redo through the far variant -> fold
+    auto emit_iteration = [&](int j1, const std::string& ind) {
+      for (int j = 0; j < j1; j++) emit_loads(j, ind.c_str());
+      for (int j = 0; j < j1; j++)
+        for (int e = 0; e < V; e++) o << ind << ctype(pre_dt) << " t" << j << "_" << e << ";\n";
+      if (trig) o << ind << "bool far = false;\n";
+      for (int j = 0; j < j1; j++) emit_values(j, ind.c_str(), false);
+      if (trig) {
+        o << ind << "if (__builtin_expect(far, 0)) {\n";
+        for (int j = 0; j < j1; j++) emit_values(j, (ind + "  ").c_str(), true);
+        o << ind << "}\n";
+      }
+      for (int j = 0; j < j1; j++)
+        for (int e = 0; e < V; e++) o << ind << "acc = WKF_FOLD((float)t" << j << "_" << e << ", acc);\n";
+    };
+    o << "  u32 k = t;\n";
+    if (U > 1) {
+      o << "  for (; k + " << (U - 1) * T << "u < a.nvec; k += " << U * T << "u) {\n";
+      emit_iteration(U, "    ");
+      o << "  }\n";
+    }
+    o << "  for (; k < a.nvec; k += " << T << "u) {\n";
+    emit_iteration(1, "    ");
+    o << "  }\n";
+    if (T > 1) o << "  acc = wkf_lanes_fold<" << std::min(T, 64) << ">(acc);\n";
+    if (T > 64) {
+      const int WPR = T / 64;  // waves per row
+      o << "  if ((threadIdx.x & 63u) == 0u) wkf_partial[threadIdx.x >> 6] = acc;\n";
+      o << "  __syncthreads();\n";
+      o << "  const u32 first_wave = (threadIdx.x / " << T << "u) * " << WPR << "u;\n";
+      o << "  acc = wkf_partial[first_wave];\n";
+      o << "  for (u32 w = 1; w < " << WPR << "u; w++) acc = WKF_FOLD(wkf_partial[first_wave + w], acc);\n";
+    }
+    o << "  if (live && t == 0u) " << out_ptr << "[" << base_expr(N) << "] = " << store_value << ";\n";
+    o << "}\n";
+  } else {
+    const int W = s.waves;
+    o << "extern \"C\" __global__ void __launch_bounds__(" << 64 * W << ") wkf_kernel(const Args a) {\n";
+    if (W > 1) o << "  __shared__ float wkf_partial[" << W << "][64];\n";
+    o << "  const u32 lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;\n";
+    // The 64 lanes of a wave sit on 64 neighbouring positions of the LAST outer dim.
+    if (Ro == 0) {
+      o << "  const bool live = lane == 0u && blockIdx.x == 0u;\n";
+    } else {
+      o << "  const u32 ntile = (a.oshape[" << Ro - 1 << "] + 63u) / 64u;\n";
+      o << "  const u32 col = (blockIdx.x % ntile) * 64u + lane;\n";
+      o << "  const bool live = col < a.oshape[" << Ro - 1 << "];\n";
+      o << "  const u32 i" << Ro - 1 << " = live ? col : 0u;\n";
+      if (Ro > 1) {
+        o << "  u32 rem = blockIdx.x / ntile;\n";
+        for (int d = Ro - 2; d > 0; d--)
+          o << "  const u32 i" << d << " = rem % a.oshape[" << d << "]; rem /= a.oshape[" << d << "];\n";
+        o << "  const u32 i0 = rem;\n";
+      }
+    }
+    for (int k = 0; k < N; k++)
+      o << "  const " << ctype(s.in[k].dtype) << "* q" << k << " = " << ptr(k) << " + (" << base_expr(k) << ");\n";
+    o << "  float acc = WKF_SEED;\n";
+    o << "  for (u32 k = wave; k < a.n; k += " << W << "u) {\n";
+    {
+      const bool trig = uses_trig(s.pre, s.math_pre);
+      std::ostringstream call;
+      for (int k = 0; k < N; k++) call << "q" << k << "[k * a.astride[" << k << "]], ";
+      call << "a.c";
+      if (trig) o << "    bool far = false;\n";
+      o << "    " << ctype(pre_dt) << " t = wkf_pre(" << call.str() << (trig ? ", far" : "") << ");\n";
+      if (trig) o << "    if (__builtin_expect(far, 0)) t = wkf_pre_far(" << call.str() << ");\n";
+      o << "    acc = WKF_FOLD((float)t, acc);\n  }\n";
+    }
+    if (W > 1) {
+      o << "  wkf_partial[wave][lane] = acc;\n  __syncthreads();\n";
+      o << "  if (wave == 0u) {\n";
+      o << "    for (u32 w = 1; w < " << W << "u; w++) acc = WKF_FOLD(wkf_partial[w][lane], acc);\n";
+      o << "    if (live) " << out_ptr << "[" << base_expr(N) << "] = " << store_value << ";\n  }\n";
+    } else {
+      o << "  if (live) " << out_ptr << "[" << base_expr(N) << "] = " << store_value << ";\n";
+    }
+    o << "}\n";
+  }
+  return o.str();
+}
+
+std::vector<unsigned char> reduce_pack_args(const ReduceSpec& s, const ReduceArgs& a) {
+  const size_t N = s.in.size();
+  const size_t Ro = size_t(s.outer_rank);
+  if (a.ptrs.size() != N + 1 || a.oshape.size() != Ro || a.offsets.size() != N + 1 || a.ostrides.size() != N + 1 ||
+      a.astrides.size() != N)
+    throw Error(WKF_ERR_INVALID_ARG, "reduce_pack_args: argument arity does not match the kernel");
+  std::vector<unsigned char> b;
+  for (void* p : a.ptrs) putp(b, p);
+  put32(b, a.nrows);
+  put32(b, a.n);
+  put32(b, s.shape == ReduceShape::Row ? a.n / uint32_t(s.vec) : a.n);
+  for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? a.oshape[d] : 1);
+  for (uint32_t v : a.offsets) put32(b, v);
+  for (const auto& st : a.ostrides) {
+    if (st.size() != Ro) throw Error(WKF_ERR_INVALID_ARG, "reduce_pack_args: stride rank mismatch");
+    for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? st[d] : 0);
+  }
+  for (size_t k = 0; k < std::max<size_t>(1, N); k++) put32(b, k < N ? a.astrides[k] : 0);
+  size_t nc = std::max<size_t>(1, s.pre.consts.size() + s.post.consts.size());
+  for (size_t i = 0; i < nc; i++) putf(b, i < a.consts.size() ? a.consts[i] : 0.f);
+  pad8(b);
+  return b;
+}
+
+}  // namespace wkf

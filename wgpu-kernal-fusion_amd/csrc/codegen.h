@@ -1,0 +1,122 @@
+// Kernel generator: turns a fused-kernel description into HIP source for gfx950
+// plus the signature the code-object cache is keyed by.  It replaces the WGSL
+// assembler of the reference (GenericKernel, src/kernel.rs:19-496, and
+// VisitTiledKernel, src/visit_tiled.rs:10-194).  Shapes, strides, offsets and
+// literal constants are kernel ARGUMENTS, so one binary serves every tensor size
+// and every constant value of the same fused structure.
+#pragma once
+
+#include <string>
+#include <vector>
+
+#include "core.h"
+
+namespace wkf {
+
+// ---- map kernels: out[i] = expr(in_0[i], ..., in_{n-1}[i]) -----------------
+// Covers the reference's element-wise, pair-wise, resize and slice_assign
+// kernels (K1, K2, K5, K6: src/visit_tiled.rs:80-144, src/resize.rs:43-88,
+// src/slice_assign.rs:49-66).
+struct MapOperandSpec {
+  DType dtype;
+  bool linear;       // index = offset + work_item * V (contiguous over the iteration space)
+  int inner_stride;  // vector mode: 0 or 1 (compile-time); scalar mode: -1 = run-time value
+};
+
+// Which implementation a transcendental op gets.
+//  Stored: the kernel's values are stored as they are.  An op whose value feeds
+//          another op ("interior") is evaluated with an f64 core and rounded
+//          once, so it matches the correctly rounded f32 value and later ops
+//          cannot amplify an error; the LAST op of the chain may be off by the
+//          f32 library's <= 1-2 ulp, which nothing amplifies.
+//  Folded: the values only feed a sum / product / max / min (tolerance class
+//          1e-5 relative): every op uses the f32 library.
+//  Exact:  every op is evaluated with an f64 core.
+enum class MathPolicy : int { Stored = 0, Folded = 1, Exact = 2 };
+
+struct MapSpec {
+  int rank;                          // rank of the coalesced iteration space (1..kMaxRank)
+  int vec;                           // elements per work item: 1, 2, 4 or 8
+  int unroll;                        // work items per thread
+  bool nontemporal;                  // streaming loads/stores bypass cache allocation
+  std::vector<MapOperandSpec> in;    // inputs
+  MapOperandSpec out;
+  Program prog;
+  MathPolicy math = MathPolicy::Stored;
+};
+constexpr int kMaxRank = 6;
+constexpr int kMapBlock = 256;
+
+std::string map_signature(const MapSpec& s);
+std::string map_source(const MapSpec& s);
+// Size in bytes of the argument block and the packer that fills it.
+struct MapArgs {
+  std::vector<void*> ptrs;               // inputs..., out
+  uint32_t nwork;                        // number of work items (vectors)
+  std::vector<uint32_t> shape;           // coalesced shape; the last entry is in work items
+  std::vector<uint32_t> offsets;         // per operand, elements
+  std::vector<std::vector<uint32_t>> strides;  // per operand, per dim, elements
+  std::vector<float> consts;
+};
+std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a);
+
+// ---- reduce kernels -----------------------------------------------------------
+// K3 of the reference (src/reduce.rs:83-281) re-designed: `Row` puts T
+// consecutive lanes on one output element and walks the axis with coalesced
+// vector loads; `Col` puts the 64 lanes of a wave on 64 neighbouring outputs and
+// walks the axis in the waves of the block.
+enum class ReduceShape { Row, Col };
+
+struct ReduceOperandSpec {
+  DType dtype;
+  int axis_stride;  // Row: 0 or 1 (compile time).  Col: -1 = run-time value
+};
+
+struct ReduceSpec {
+  ReduceShape shape;
+  int outer_rank;                 // 0..3 dims of the output iteration space (coalesced)
+  int vec;                        // Row: elements per load along the axis
+  int threads_per_row;            // Row: T (power of two, 1..1024)
+  int block;                      // threads per block
+  int unroll;                     // Row: independent loads in flight per operand
+  int waves;                      // Col: waves per block walking the axis
+  ReduceOp rop;
+  std::vector<ReduceOperandSpec> in;
+  DType out_dtype;
+  Program pre;                    // value fed to the fold (one per axis element)
+  Program post;                   // applied once to the folded value; one Load of operand 0 = the folded value
+  MathPolicy math_pre = MathPolicy::Folded;
+  MathPolicy math_post = MathPolicy::Stored;
+};
+
+std::string reduce_signature(const ReduceSpec& s);
+std::string reduce_source(const ReduceSpec& s);
+struct ReduceArgs {
+  std::vector<void*> ptrs;                        // inputs..., out
+  uint32_t nrows;                                 // number of outputs
+  uint32_t n;                                     // axis length (elements)
+  std::vector<uint32_t> oshape;                   // outer shape
+  std::vector<uint32_t> offsets;                  // per operand incl. out
+  std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. out, per outer dim
+  std::vector<uint32_t> astrides;                 // per input
+  std::vector<float> consts;                      // pre consts then post consts
+};
+std::vector<unsigned char> reduce_pack_args(const ReduceSpec& s, const ReduceArgs& a);
+
+// ---- GEMM ----------------------------------------------------------------------
+// K4 of the reference (src/matmul.rs:56-155) re-designed for MFMA.
+struct GemmSpec {
+  DType dtype;       // A, B and C share it (src/matmul.rs:157-183)
+  int tile_m, tile_n, tile_k;
+  int waves_m, waves_n;
+  bool exact_tiles;  // M, N, K are multiples of the tile: no edge handling
+};
+std::string gemm_signature(const GemmSpec& s);
+std::string gemm_source(const GemmSpec& s);
+struct GemmArgs {
+  const void* a; const void* b; void* c;
+  uint32_t m, n, k;
+};
+std::vector<unsigned char> gemm_pack_args(const GemmArgs& a);
+
+}  // namespace wkf

@@ -1,0 +1,591 @@
+#include "graph.h"
+
+#include <algorithm>
+#include <functional>
+#include <mutex>
+#include <set>
+#include <unordered_map>
+#include <sstream>
+
+namespace wkf {
+
+namespace {
+
+void check(int rc) {
+  if (rc != WKF_OK) throw Error(rc, wkf_last_error());
+}
+
+uint32_t to_u32(size_t v, const char* what) {
+  if (v > 0xffffffffull) throw Error(WKF_ERR_UNSUPPORTED, std::string(what) + " does not fit 32-bit indexing");
+  return uint32_t(v);
+}
+
+int pow2_ceil(size_t v) {
+  int p = 1;
+  while (size_t(p) < v) p <<= 1;
+  return p;
+}
+
+// The iteration space of one kernel seen by all of its operands at once:
+// `shape` plus one stride vector per operand.  Dimensions of size 1 are dropped
+// and neighbouring dimensions are merged when every operand walks them as one.
+struct Space {
+  std::vector<size_t> shape;
+  std::vector<std::vector<size_t>> strides;  // [operand][dim]
+};
+
+Space coalesce(const std::vector<size_t>& shape, const std::vector<std::vector<size_t>>& strides) {
+  Space s;
+  s.strides.resize(strides.size());
+  for (size_t d = 0; d < shape.size(); d++) {
+    if (shape[d] == 1) continue;
+    bool merged = false;
+    if (!s.shape.empty()) {
+      bool ok = true;
+      for (size_t k = 0; k < strides.size(); k++) ok &= s.strides[k].back() == shape[d] * strides[k][d];
+      if (ok) {
+        s.shape.back() *= shape[d];
+        for (size_t k = 0; k < strides.size(); k++) s.strides[k].back() = strides[k][d];
+        merged = true;
+      }
+    }
+    if (!merged) {
+      s.shape.push_back(shape[d]);
+      for (size_t k = 0; k < strides.size(); k++) s.strides[k].push_back(strides[k][d]);
+    }
+  }
+  return s;
+}
+
+std::string dims(const std::vector<size_t>& v) {
+  std::ostringstream o;
+  o << '[';
+  for (size_t i = 0; i < v.size(); i++) o << (i ? "," : "") << v[i];
+  o << ']';
+  return o.str();
+}
+
+void* element_ptr(const TensorData& td) { return wkf_buffer_ptr(td.buffer.get()); }
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+
+int Resolver::ExprBuilder::load(const TensorData& td) {
+  for (size_t k = 0; k < operands.size(); k++) {
+    if (operands[k].buffer.get() == td.buffer.get() && operands[k].dtype == td.dtype && operands[k].layout == td.layout)
+      return operand_value[k];
+  }
+  operands.push_back(td);
+  Instr in;
+  in.op = Op::Load;
+  in.dtype = td.dtype;
+  in.operand = int(operands.size()) - 1;
+  prog.ins.push_back(in);
+  operand_value.push_back(int(prog.ins.size()) - 1);
+  return operand_value.back();
+}
+
+int Resolver::ExprBuilder::emit(Op op, int a, int b, DType dt, bool has_const, float c) {
+  Instr in;
+  in.op = op;
+  in.a = a;
+  in.b = b;
+  in.dtype = dt;
+  if (has_const) {
+    in.cslot = int(prog.consts.size());
+    prog.consts.push_back(c);
+  }
+  prog.ins.push_back(in);
+  return int(prog.ins.size()) - 1;
+}
+
+int Resolver::build(ExprBuilder& eb, const NodeP& n, int pairwise_budget) {
+  auto it = eb.memo.find(n.get());
+  if (it != eb.memo.end()) return it->second;
+  int v;
+  // Keep kernels within a sane register / argument budget: past it, a sub-tree is materialised.
+  const bool room = eb.prog.ins.size() < 48 && eb.operands.size() < 7;
+  if (n->kind == NodeKind::ElementWise) {
+    int a = build(eb, n->a, pairwise_budget);
+    v = eb.emit(n->op, a, -1, n->dtype, is_const_op(n->op), n->constant);
+  } else if (n->kind == NodeKind::PairWise && pairwise_budget > 0 && room) {
+    int a = build(eb, n->a, pairwise_budget - 1);
+    int b = build(eb, n->b, pairwise_budget - 1);
+    v = eb.emit(n->op, a, b, n->dtype, false, 0.f);
+  } else {
+    TensorData td = resolve(n);
+    v = eb.load(td);
+  }
+  eb.memo[n.get()] = v;
+  return v;
+}
+
+TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero) {
+  TensorData td;
+  td.device = dev_;
+  td.layout = Layout::contiguous(shape);
+  td.dtype = dt;
+  wkf_buffer* b = nullptr;
+  // padded_tensor_size, src/tensor.rs:775-783: a multiple of 4 bytes, at least 4.
+  size_t bytes = std::max<size_t>(4, (td.layout.numel() * dtype_size(dt) + 3) & ~size_t(3));
+  check(wkf_buffer_alloc(dev_, bytes, zero ? 1 : 0, &b));
+  td.buffer = BufRef(b);
+  return td;
+}
+
+extern std::mutex g_source_mu;
+extern std::unordered_map<std::string, std::string> g_sources;
+
+wkf_kernel* Resolver::kernel(const std::string& sig, const std::string& src) {
+  {
+    std::lock_guard<std::mutex> lock(g_source_mu);
+    g_sources.emplace(sig, src);
+  }
+  wkf_kernel* k = nullptr;
+  check(wkf_module_get(dev_, sig.c_str(), src.c_str(), "wkf_kernel", &k));
+  return k;
+}
+
+void Resolver::record(LaunchRecord&& r, wkf_kernel* k, const std::vector<unsigned char>& args) {
+  if (st_.timing) check(wkf_timer_create(dev_, &r.timer));
+  int rc = wkf_launch(dev_, k, r.grid, r.block, 0, args.data(), args.size(), r.timer);
+  if (rc != WKF_OK) {
+    if (r.timer) wkf_timer_destroy(r.timer);
+    throw Error(rc, wkf_last_error());
+  }
+  if (log_) log_->push_back(std::move(r));
+  else if (r.timer) wkf_timer_destroy(r.timer);
+}
+
+TensorData Resolver::resolve(const NodeP& n) {
+  auto it = materialized_.find(n.get());
+  if (it != materialized_.end()) return it->second;
+  TensorData out = resolve_uncached(n);
+  if (shared_.count(n.get()) && n->kind != NodeKind::Tensor) materialized_[n.get()] = out;
+  return out;
+}
+
+TensorData Resolver::resolve_uncached(const NodeP& n) {
+  switch (n->kind) {
+    case NodeKind::Tensor:
+      return n->data;  // a clone: the graph keeps its own reference, so a leaf is never "owned" (src/compute_graph/resolve.rs:246-248)
+    case NodeKind::ElementWise: {
+      // collect_element_wise_ops, src/compute_graph/resolve.rs:49-61
+      std::vector<const Node*> chain;
+      const Node* cur = n.get();
+      NodeP base;
+      while (cur->kind == NodeKind::ElementWise) {
+        chain.push_back(cur);
+        base = cur->a;
+        cur = cur->a.get();
+      }
+      if (base->kind == NodeKind::Reduce && !materialized_.count(base.get()))
+        return run_reduce(base, chain);  // post-fusion into the reduce, src/compute_graph/resolve.rs:72-74
+      return run_map(n);
+    }
+    case NodeKind::PairWise: return run_map(n);
+    case NodeKind::Reduce: return run_reduce(n, {});
+    case NodeKind::MatMul: return run_matmul(n);
+    case NodeKind::MapLayout: return run_map_layout(n);
+    case NodeKind::Resize: return run_resize(n);
+    case NodeKind::SliceAssign: return run_slice_assign(n);
+  }
+  invalid("resolve: unknown node kind");
+}
+
+// A node consumed by several nodes of the graph under `root` is computed once per
+// resolve and shared.  (The reference recomputes it per use, src/tensor.rs:286-288;
+// the values are identical, and because the shared copy holds a reference the
+// buffer is never reused in place.)
+TensorData Resolver::resolve_root(const NodeP& root) {
+  std::map<const Node*, int> uses;
+  std::set<const Node*>& shared = shared_;
+  shared.clear();
+  materialized_.clear();
+  std::function<void(const NodeP&)> walk = [&](const NodeP& n) {
+    if (!n) return;
+    if (++uses[n.get()] > 1) {
+      shared.insert(n.get());
+      return;
+    }
+    walk(n->a);
+    walk(n->b);
+  };
+  walk(root);
+  shared.erase(root.get());
+  TensorData out = resolve(root);
+  materialized_.clear();
+  return out;
+}
+
+TensorData Resolver::run_map(const NodeP& root) {
+  ExprBuilder eb;
+  int v = build(eb, root, pairwise_budget_for_map());
+  eb.prog.result = v;
+  const DType out_dt = eb.prog.result_dtype();
+  // In-place rule: src/element_wise.rs:98 and src/pair_wise.rs:95-107 -- the first
+  // operand of the output dtype that nobody else references and that has no
+  // stride-0 overlap is overwritten; otherwise a fresh contiguous tensor.
+  int reuse = -1;
+  for (size_t k = 0; k < eb.operands.size(); k++) {
+    const TensorData& td = eb.operands[k];
+    if (td.dtype == out_dt && td.owned() && !td.layout.allocation_overlaps()) {
+      reuse = int(k);
+      break;
+    }
+  }
+  TensorData out = reuse >= 0 ? eb.operands[reuse] : alloc(root->shape, out_dt, false);
+  launch_map(eb.prog, eb.operands, out, reuse >= 0);
+  return out;
+}
+
+void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place) {
+  const std::vector<size_t>& shape = out.layout.shape;
+  for (const TensorData& td : in)
+    if (td.layout.shape != shape)
+      invalid("operand shapes differ: " + dims(td.layout.shape) + " vs " + dims(shape));  // src/pair_wise.rs:92
+  size_t numel = out.layout.numel();
+  if (numel == 0) return;
+
+  std::vector<std::vector<size_t>> strides;
+  for (const TensorData& td : in) strides.push_back(td.layout.strides);
+  strides.push_back(out.layout.strides);
+  Space sp = coalesce(shape, strides);
+  if (sp.shape.empty()) {
+    sp.shape.push_back(1);
+    for (auto& s : sp.strides) s.push_back(1);
+  }
+  const size_t R = sp.shape.size();
+  if (R > size_t(kMaxRank)) throw Error(WKF_ERR_UNSUPPORTED, "map kernel: more than 6 non-mergeable dimensions");
+  const size_t N = in.size() + 1;
+  auto td_of = [&](size_t k) -> const TensorData& { return k < in.size() ? in[k] : out; };
+
+  // Vector width: 16 bytes of the widest element type, shrunk until every operand
+  // is either unit-stride and aligned or a broadcast along the inner dimension.
+  size_t max_elem = 2;
+  for (size_t k = 0; k < N; k++) max_elem = std::max(max_elem, dtype_size(td_of(k).dtype));
+  int vec = int(16 / max_elem);
+  auto vec_ok = [&](int V) {
+    if (sp.shape[R - 1] % V) return false;
+    for (size_t k = 0; k < N; k++) {
+      size_t inner = sp.strides[k][R - 1];
+      if (inner > 1) return false;
+      if (inner == 0) {
+        if (k == N - 1) return false;
+        continue;
+      }
+      if (td_of(k).layout.offset % V) return false;
+      for (size_t d = 0; d + 1 < R; d++)
+        if (sp.strides[k][d] % V) return false;
+    }
+    return true;
+  };
+  while (vec > 1 && !vec_ok(vec)) vec /= 2;
+
+  MapSpec spec;
+  spec.rank = int(R);
+  spec.vec = vec;
+  spec.prog = prog;
+  spec.math = st_.exact_math ? MathPolicy::Exact : MathPolicy::Stored;
+  const size_t nwork = numel / vec;
+  spec.unroll = nwork >= (1u << 20) ? 4 : nwork >= (1u << 16) ? 2 : 1;
+  size_t bytes = 0;
+  std::vector<size_t> cstrides = Layout::contiguous_strides(sp.shape);
+  for (size_t k = 0; k < N; k++) {
+    MapOperandSpec os;
+    os.dtype = td_of(k).dtype;
+    os.linear = sp.strides[k] == cstrides;
+    os.inner_stride = vec > 1 ? int(sp.strides[k][R - 1]) : -1;
+    if (os.linear) os.inner_stride = vec > 1 ? 1 : -1;
+    if (k < in.size()) spec.in.push_back(os);
+    else spec.out = os;
+    bytes += os.linear ? numel * dtype_size(os.dtype) : 0;
+  }
+  spec.nontemporal = bytes >= st_.nontemporal_bytes;
+
+  MapArgs args;
+  args.nwork = to_u32(nwork, "tensor size");
+  for (size_t d = 0; d < R; d++) args.shape.push_back(to_u32(d == R - 1 ? sp.shape[d] / vec : sp.shape[d], "shape"));
+  for (size_t k = 0; k < N; k++) {
+    const TensorData& td = td_of(k);
+    to_u32(td.layout.extent(), "tensor extent");
+    if (td.layout.extent() * dtype_size(td.dtype) > wkf_buffer_size(td.buffer.get()) + 3)
+      invalid("map kernel: a layout reaches past the end of its buffer");
+    args.ptrs.push_back(element_ptr(td));
+    args.offsets.push_back(to_u32(td.layout.offset, "offset"));
+    std::vector<uint32_t> st;
+    for (size_t d = 0; d < R; d++) st.push_back(to_u32(sp.strides[k][d], "stride"));
+    args.strides.push_back(st);
+  }
+  args.consts = prog.consts;
+
+  std::string sig = map_signature(spec);
+  wkf_kernel* k = kernel(sig, map_source(spec));
+  LaunchRecord r;
+  r.kind = "map";
+  r.signature = sig;
+  r.in_place = in_place;
+  size_t per_block = size_t(kMapBlock) * spec.unroll;
+  r.grid[0] = to_u32((nwork + per_block - 1) / per_block, "grid");
+  r.block[0] = kMapBlock;
+  std::ostringstream d;
+  d << "shape=" << dims(sp.shape) << " vec=" << vec << " unroll=" << spec.unroll << " operands=" << N
+    << (in_place ? " in_place" : "");
+  r.detail = d.str();
+  record(std::move(r), k, map_pack_args(spec, args));
+}
+
+TensorData Resolver::make_contiguous(const TensorData& td) {
+  if (td.layout.is_contiguous()) return td;
+  TensorData out = alloc(td.layout.shape, td.dtype, false);
+  Program p;
+  Instr in;
+  in.op = Op::Load;
+  in.dtype = td.dtype;
+  in.operand = 0;
+  p.ins.push_back(in);
+  p.result = 0;
+  launch_map(p, {td}, out, false);
+  return out;
+}
+
+TensorData Resolver::run_reduce(const NodeP& rn, const std::vector<const Node*>& post_chain) {
+  ExprBuilder eb;
+  int v = build(eb, rn->a, pairwise_budget_for_reduce());
+  eb.prog.result = v;
+  const DType pre_dt = eb.prog.result_dtype();
+  // post: the chain above the reduce, innermost first (src/compute_graph/resolve.rs:164-196)
+  Program post;
+  {
+    Instr ld;
+    ld.op = Op::Load;
+    ld.dtype = pre_dt;
+    ld.operand = 0;
+    post.ins.push_back(ld);
+    int cur = 0;
+    for (size_t i = post_chain.size(); i-- > 0;) {
+      const Node* c = post_chain[i];
+      Instr in;
+      in.op = c->op;
+      in.a = cur;
+      in.dtype = c->dtype;
+      if (is_const_op(c->op)) {
+        in.cslot = int(post.consts.size());
+        post.consts.push_back(c->constant);
+      }
+      post.ins.push_back(in);
+      cur = int(post.ins.size()) - 1;
+    }
+    post.result = cur;
+  }
+  const std::vector<size_t>& shape = rn->a->shape;
+  const size_t axis = rn->axis;
+  if (axis >= shape.size()) invalid("reduce: axis out of range");
+  for (const TensorData& td : eb.operands)
+    if (td.layout.shape != shape) invalid("reduce: operand shapes differ");
+  std::vector<size_t> out_shape;
+  for (size_t d = 0; d < shape.size(); d++)
+    if (d != axis) out_shape.push_back(shape[d]);
+  TensorData out = alloc(out_shape, post.result_dtype(), false);
+  const size_t nrows = out.layout.numel();
+  const size_t n = shape[axis];
+  if (nrows == 0) return out;
+
+  const size_t N = eb.operands.size();
+  std::vector<std::vector<size_t>> ostr;
+  for (const TensorData& td : eb.operands) {
+    std::vector<size_t> s;
+    for (size_t d = 0; d < shape.size(); d++)
+      if (d != axis) s.push_back(td.layout.strides[d]);
+    ostr.push_back(s);
+  }
+  ostr.push_back(out.layout.strides);
+  Space sp = coalesce(out_shape, ostr);
+  const size_t Ro = sp.shape.size();
+  if (Ro > 3) throw Error(WKF_ERR_UNSUPPORTED, "reduce kernel: more than 3 non-mergeable outer dimensions");
+
+  ReduceSpec spec;
+  spec.outer_rank = int(Ro);
+  spec.rop = rn->rop;
+  spec.out_dtype = post.result_dtype();
+  spec.pre = eb.prog;
+  spec.post = post;
+  spec.math_pre = st_.exact_math ? MathPolicy::Exact : MathPolicy::Folded;
+  spec.math_post = st_.exact_math ? MathPolicy::Exact : MathPolicy::Stored;
+  spec.vec = 1;
+  spec.threads_per_row = 1;
+  spec.block = 256;
+  spec.unroll = 1;
+  spec.waves = 1;
+  bool row = true;
+  for (const TensorData& td : eb.operands) row &= (n <= 1 || td.layout.strides[axis] <= 1);
+  spec.shape = row ? ReduceShape::Row : ReduceShape::Col;
+
+  LaunchRecord r;
+  std::ostringstream d;
+  if (row) {
+    size_t max_elem = 2;
+    for (const TensorData& td : eb.operands) max_elem = std::max(max_elem, dtype_size(td.dtype));
+    int vec = int(16 / max_elem);
+    auto vec_ok = [&](int V) {
+      if (n % V) return false;
+      for (size_t k = 0; k < N; k++) {
+        const TensorData& td = eb.operands[k];
+        if (td.layout.strides[axis] == 0) continue;
+        if (td.layout.offset % V) return false;
+        for (size_t dd = 0; dd < Ro; dd++)
+          if (sp.strides[k][dd] % V) return false;
+      }
+      return true;
+    };
+    while (vec > 1 && !vec_ok(vec)) vec /= 2;
+    spec.vec = vec;
+    const size_t nvec = n / vec;
+    // About eight vector loads per lane; more lanes per row when there are too few rows to fill the chip.
+    int T = std::min(1024, pow2_ceil((nvec + 7) / 8));
+    wkf_props props;
+    check(wkf_device_props(dev_, &props));
+    const size_t want_threads = size_t(props.compute_units) * 1024;
+    while (T < 1024 && size_t(T) * 2 <= nvec && nrows * T < want_threads) T *= 2;
+    spec.threads_per_row = T;
+    spec.block = std::max(256, T);
+    size_t per_lane = (nvec + T - 1) / T;
+    spec.unroll = per_lane >= 4 ? 4 : per_lane >= 2 ? 2 : 1;
+    for (const TensorData& td : eb.operands)
+      spec.in.push_back({td.dtype, (n <= 1 || td.layout.strides[axis] == 0) ? 0 : 1});
+    size_t rpb = size_t(spec.block / T);
+    r.grid[0] = to_u32((nrows + rpb - 1) / rpb, "grid");
+    r.block[0] = uint32_t(spec.block);
+    r.kind = "red_row";
+    d << "rows=" << nrows << " n=" << n << " vec=" << vec << " threads_per_row=" << T << " unroll=" << spec.unroll;
+  } else {
+    spec.waves = n >= 64 ? 16 : n >= 8 ? 4 : 1;
+    for (const TensorData& td : eb.operands) spec.in.push_back({td.dtype, -1});
+    size_t lanes_dim = Ro ? sp.shape[Ro - 1] : 1;
+    size_t rest = nrows / lanes_dim;
+    r.grid[0] = to_u32(((lanes_dim + 63) / 64) * rest, "grid");
+    r.block[0] = uint32_t(64 * spec.waves);
+    r.kind = "red_col";
+    d << "outputs=" << nrows << " n=" << n << " waves=" << spec.waves;
+  }
+
+  ReduceArgs args;
+  args.nrows = to_u32(nrows, "output size");
+  args.n = to_u32(n, "axis length");
+  for (size_t dd = 0; dd < Ro; dd++) args.oshape.push_back(to_u32(sp.shape[dd], "shape"));
+  for (size_t k = 0; k <= N; k++) {
+    const TensorData& td = k < N ? eb.operands[k] : out;
+    to_u32(td.layout.extent(), "tensor extent");
+    args.ptrs.push_back(element_ptr(td));
+    args.offsets.push_back(to_u32(td.layout.offset, "offset"));
+    std::vector<uint32_t> st;
+    for (size_t dd = 0; dd < Ro; dd++) st.push_back(to_u32(sp.strides[k][dd], "stride"));
+    args.ostrides.push_back(st);
+    if (k < N) args.astrides.push_back(to_u32(td.layout.strides[axis], "stride"));
+  }
+  args.consts = eb.prog.consts;
+  args.consts.insert(args.consts.end(), post.consts.begin(), post.consts.end());
+
+  std::string sig = reduce_signature(spec);
+  wkf_kernel* k = kernel(sig, reduce_source(spec));
+  r.signature = sig;
+  r.detail = d.str();
+  record(std::move(r), k, reduce_pack_args(spec, args));
+  return out;
+}
+
+TensorData Resolver::run_map_layout(const NodeP& n) {
+  // MapLayoutOperation::run, src/map_layout.rs:26-39: a view on the same buffer.
+  TensorData in = resolve(n->a);
+  TensorData out = in;
+  const Layout& l = in.layout;
+  switch (n->map_kind) {
+    case MapKind::Slice: out.layout = l.slice(n->ranges); break;
+    case MapKind::Transpose:
+      std::swap(out.layout.shape[n->axis0], out.layout.shape[n->axis1]);
+      std::swap(out.layout.strides[n->axis0], out.layout.strides[n->axis1]);
+      break;
+    case MapKind::Broadcast: {
+      // one stride-0 dimension inserted at axis0, src/map_layout.rs:69-98
+      Layout b;
+      b.offset = l.offset;
+      b.shape = n->new_shape;
+      for (size_t i = 0; i <= l.rank(); i++) {
+        if (i == n->axis0) b.strides.push_back(0);
+        if (i < l.rank()) b.strides.push_back(l.strides[i]);
+      }
+      out.layout = b;
+      break;
+    }
+  }
+  return out;
+}
+
+TensorData Resolver::run_resize(const NodeP& n) {
+  const std::vector<size_t>& in_shape = n->a->shape;
+  const bool is_reshape = n->fill_shape == n->new_shape && in_shape != n->new_shape;
+  ExprBuilder eb;
+  if (st_.fusion == FusionMode::Tree) {
+    eb.prog.result = build(eb, n->a, pairwise_budget_for_map());
+  } else {
+    eb.prog.result = eb.load(resolve(n->a));
+  }
+  const DType dt = eb.prog.result_dtype();
+  if (is_reshape || in_shape == n->new_shape) {
+    // reshape (src/resize.rs:131-144): a dense copy in the input's own index order;
+    // the contiguous result is then read with the new shape.
+    TensorData out = alloc(in_shape, dt, false);
+    launch_map(eb.prog, eb.operands, out, false);
+    out.layout = Layout::contiguous(n->new_shape);
+    return out;
+  }
+  // resize (src/resize.rs:121-129): the input lands in the [0, in_shape) corner of a
+  // zero-filled tensor of the new shape (wgpu zero-initialises, hipMalloc does not).
+  // Where the new shape is smaller than the input the copy is cropped.
+  if (in_shape.size() != n->new_shape.size()) invalid("resize: rank must not change");
+  std::vector<std::pair<size_t, size_t>> corner;
+  bool pad = false;
+  for (size_t d = 0; d < in_shape.size(); d++) {
+    corner.push_back({0, std::min(in_shape[d], n->new_shape[d])});
+    pad |= n->new_shape[d] > in_shape[d];
+  }
+  TensorData out = alloc(n->new_shape, dt, pad);
+  TensorData view = out;
+  view.layout = out.layout.slice(corner);
+  std::vector<TensorData> ops = eb.operands;
+  for (TensorData& td : ops) td.layout = td.layout.slice(corner);
+  launch_map(eb.prog, ops, view, false);
+  return out;
+}
+
+TensorData Resolver::run_slice_assign(const NodeP& n) {
+  TensorData target = resolve(n->a);
+  if (!target.owned() || target.layout.allocation_overlaps()) {
+    // The reference writes into the target's buffer whoever else holds it
+    // (src/slice_assign.rs:68-72), which can change a tensor the caller still
+    // uses.  A shared target is copied first.
+    TensorData copy = alloc(target.layout.shape, target.dtype, false);
+    Program p;
+    Instr ld;
+    ld.op = Op::Load;
+    ld.dtype = target.dtype;
+    ld.operand = 0;
+    p.ins.push_back(ld);
+    p.result = 0;
+    launch_map(p, {target}, copy, false);
+    target = copy;
+  }
+  ExprBuilder eb;
+  if (st_.fusion == FusionMode::Tree) eb.prog.result = build(eb, n->b, pairwise_budget_for_map());
+  else eb.prog.result = eb.load(resolve(n->b));
+  if (eb.prog.result_dtype() != target.dtype) invalid("slice_assign: dtype mismatch");
+  TensorData view = target;
+  view.layout = target.layout.slice(n->ranges);
+  if (view.layout.shape != n->b->shape)
+    invalid("slice_assign: value shape " + dims(n->b->shape) + " does not match the slice " + dims(view.layout.shape));  // src/slice_assign.rs:69
+  launch_map(eb.prog, eb.operands, view, true);
+  return target;
+}
+
+}  // namespace wkf

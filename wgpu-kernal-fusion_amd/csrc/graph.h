@@ -1,0 +1,79 @@
+// The executor of the lazy graph: walks a node, applies the fusion rules and
+// plans + launches one generated kernel per fused group.  Restates
+// ComputeGraphInner::resolve and its helpers (src/compute_graph/resolve.rs:16-248)
+// and the run_with_query methods of the reference's kernel objects.
+#pragma once
+
+#include <map>
+#include <set>
+#include <string>
+#include <vector>
+
+#include "codegen.h"
+#include "core.h"
+
+namespace wkf {
+
+// One kernel launch of a resolve; the analogue of a PerformanceQueries entry in
+// the reference's timing map (src/compute_graph/mod.rs:275).
+struct LaunchRecord {
+  std::string kind;        // map | red_row | red_col | gemm
+  std::string signature;   // cache key of the kernel
+  std::string detail;      // human-readable launch geometry
+  wkf_timer* timer = nullptr;
+  uint32_t grid[3] = {1, 1, 1};
+  uint32_t block[3] = {1, 1, 1};
+  bool in_place = false;
+};
+
+struct Settings {
+  FusionMode fusion = FusionMode::Tree;
+  bool timing = true;             // record a hipEvent pair around every launch
+  bool exact_math = false;        // every transcendental through an f64 core (MathPolicy::Exact)
+  size_t nontemporal_bytes = size_t(32) << 20;  // map kernels moving at least this much use streaming loads/stores
+};
+
+class Resolver {
+ public:
+  Resolver(wkf_device* dev, const Settings& st, std::vector<LaunchRecord>* log) : dev_(dev), st_(st), log_(log) {}
+  // Entry point: materialise `root` (ComputeGraph::resolve, src/compute_graph/mod.rs:241-248).
+  TensorData resolve_root(const NodeP& root);
+
+ private:
+  TensorData resolve(const NodeP& n);
+  TensorData resolve_uncached(const NodeP& n);
+  struct ExprBuilder {
+    Program prog;
+    std::vector<TensorData> operands;
+    std::map<const Node*, int> memo;
+    std::vector<int> operand_value;  // value id of the Load of operand k
+    int load(const TensorData& td);
+    int emit(Op op, int a, int b, DType dt, bool has_const, float c);
+  };
+
+  int build(ExprBuilder& eb, const NodeP& n, int pairwise_budget);
+  int pairwise_budget_for_map() const { return st_.fusion == FusionMode::Tree ? 1 << 20 : 1; }
+  int pairwise_budget_for_reduce() const { return st_.fusion == FusionMode::Tree ? 1 << 20 : 0; }
+
+  TensorData run_map(const NodeP& root);
+  TensorData run_reduce(const NodeP& reduce, const std::vector<const Node*>& post_chain);
+  TensorData run_matmul(const NodeP& n);
+  TensorData run_map_layout(const NodeP& n);
+  TensorData run_resize(const NodeP& n);
+  TensorData run_slice_assign(const NodeP& n);
+
+  // out[i] = prog(operands[i]) over out.layout.shape; every operand layout has that shape.
+  void launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
+  TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero);
+  TensorData make_contiguous(const TensorData& td);
+  void record(LaunchRecord&& r, wkf_kernel* k, const std::vector<unsigned char>& args);
+  wkf_kernel* kernel(const std::string& sig, const std::string& src);
+
+  wkf_device* dev_;
+  Settings st_;
+  std::vector<LaunchRecord>* log_;
+  std::set<const Node*> shared_;
+  std::map<const Node*, TensorData> materialized_;  // nodes with several consumers, computed once per resolve
+};
+
+}  // namespace wkf

@@ -1,0 +1,531 @@
+// Level 0 of the C ABI (include/wkf_hip.h): the only host translation unit that
+// touches the HIP runtime or hiprtc.  Everything above it (layouts, the lazy
+// graph, the fusion pass, the kernel generator) is device-agnostic C++ and
+// reaches the GPU only through these entry points.
+#include "wkf_hip.h"
+
+#include <hip/hip_runtime.h>
+#include <hip/hiprtc.h>
+
+#include <dlfcn.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <atomic>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+namespace {
+
+thread_local std::string g_last_error;
+
+int fail(int code, const std::string& msg) {
+  g_last_error = msg;
+  return code;
+}
+
+#define WKF_HIP_CHECK(expr)                                                        \
+  do {                                                                             \
+    hipError_t e_ = (expr);                                                        \
+    if (e_ != hipSuccess)                                                          \
+      return fail(e_ == hipErrorOutOfMemory ? WKF_ERR_OOM : WKF_ERR_HIP,           \
+                  std::string(#expr) + ": " + hipGetErrorString(e_));              \
+  } while (0)
+
+// Options every kernel is compiled with.  -ffp-contract=off keeps each fused op
+// rounded on its own (no cross-op FMA); packed-fp32 code generation is disabled.
+const char* const kCompileOptions[] = {
+    "--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-std=c++17",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+};
+constexpr int kNumCompileOptions = sizeof(kCompileOptions) / sizeof(kCompileOptions[0]);
+// Bump when the meaning of a cached code object changes for reasons the source text does not show.
+const char* const kCacheVersion = "wkf-cache-1";
+
+uint64_t fnv1a(const void* data, size_t n, uint64_t h = 1469598103934665603ull) {
+  const unsigned char* p = static_cast<const unsigned char*>(data);
+  for (size_t i = 0; i < n; i++) {
+    h ^= p[i];
+    h *= 1099511628211ull;
+  }
+  return h;
+}
+
+std::string library_dir() {
+  Dl_info info;
+  if (dladdr(reinterpret_cast<void*>(&library_dir), &info) && info.dli_fname) {
+    std::string p(info.dli_fname);
+    size_t slash = p.rfind('/');
+    if (slash != std::string::npos) return p.substr(0, slash);
+  }
+  return ".";
+}
+
+std::string cache_dir() {
+  const char* env = getenv("WKF_CACHE_DIR");
+  std::string d = env && *env ? std::string(env) : library_dir() + "/kcache";
+  mkdir(d.c_str(), 0755);
+  return d;
+}
+
+size_t pool_bucket(size_t bytes) {
+  if (bytes < 256) bytes = 256;
+  if (bytes <= (1u << 20)) {
+    size_t b = 256;
+    while (b < bytes) b <<= 1;
+    return b;
+  }
+  const size_t mib = 1u << 20;
+  return (bytes + mib - 1) / mib * mib;
+}
+
+}  // namespace
+
+struct wkf_kernel {
+  hipModule_t module = nullptr;
+  hipFunction_t function = nullptr;
+  std::string signature;
+  std::string entry;
+};
+
+struct wkf_device {
+  int ordinal = -1;
+  bool planner = false;
+  hipStream_t stream = nullptr;
+  std::recursive_mutex mu;
+  std::unordered_map<std::string, wkf_kernel*> kernels;
+  std::map<size_t, std::vector<void*>> pool;  // capacity -> free device pointers
+  size_t pool_bytes = 0;
+  size_t pool_limit = size_t(96) << 30;
+  uint64_t n_compiled = 0, n_disk = 0, n_mem = 0;
+  std::string cache_path;
+  wkf_props props{};
+};
+
+struct wkf_buffer {
+  wkf_device* dev;
+  void* ptr;
+  size_t bytes;
+  size_t capacity;
+  std::atomic<int> refs;
+  bool host_valid;  // plan-only devices: true once the host has uploaded contents
+};
+
+struct wkf_timer {
+  wkf_device* dev;
+  hipEvent_t begin = nullptr, end = nullptr;
+  bool recorded = false;
+};
+
+// Lets the layers above this file leave their message where wkf_last_error() finds it.
+void wkf_set_last_error_(const char* msg) { g_last_error = msg ? msg : ""; }
+
+extern "C" {
+
+const char* wkf_last_error(void) { return g_last_error.c_str(); }
+
+int wkf_device_create(int ordinal, wkf_device** out) {
+  if (!out || ordinal < 0) return fail(WKF_ERR_INVALID_ARG, "wkf_device_create: bad arguments");
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= ordinal)
+    return fail(WKF_ERR_NO_DEVICE, "wkf_device_create: no HIP device with ordinal " +
+                                       std::to_string(ordinal) + " (" +
+                                       (e != hipSuccess ? hipGetErrorString(e) : "count too small") + ")");
+  WKF_HIP_CHECK(hipSetDevice(ordinal));
+  wkf_device* d = new wkf_device();
+  d->ordinal = ordinal;
+  hipError_t se = hipStreamCreateWithFlags(&d->stream, hipStreamNonBlocking);
+  if (se != hipSuccess) {
+    delete d;
+    return fail(WKF_ERR_HIP, std::string("hipStreamCreateWithFlags: ") + hipGetErrorString(se));
+  }
+  hipDeviceProp_t p;
+  if (hipGetDeviceProperties(&p, ordinal) == hipSuccess) {
+    d->props.ordinal = ordinal;
+    d->props.compute_units = p.multiProcessorCount;
+    d->props.wave_size = p.warpSize;
+    d->props.max_threads_per_block = p.maxThreadsPerBlock;
+    d->props.clock_khz = p.clockRate;
+    d->props.lds_bytes_per_block = p.sharedMemPerBlock;
+    d->props.total_mem_bytes = p.totalGlobalMem;
+    snprintf(d->props.arch, sizeof(d->props.arch), "%s", p.gcnArchName);
+  }
+  if (strncmp(d->props.arch, "gfx950", 6) != 0) {
+    std::string arch = d->props.arch;
+    hipStreamDestroy(d->stream);
+    delete d;
+    return fail(WKF_ERR_UNSUPPORTED, "wkf_device_create: kernels are written for gfx950, device is " + arch);
+  }
+  d->cache_path = cache_dir();
+  *out = d;
+  return WKF_OK;
+}
+
+int wkf_device_create_planner(wkf_device** out) {
+  if (!out) return fail(WKF_ERR_INVALID_ARG, "wkf_device_create_planner: null out");
+  wkf_device* d = new wkf_device();
+  d->planner = true;
+  d->props.ordinal = -1;
+  d->props.compute_units = 256;
+  d->props.wave_size = 64;
+  d->props.max_threads_per_block = 1024;
+  d->props.clock_khz = 2400000;
+  d->props.lds_bytes_per_block = 160 * 1024;
+  d->props.total_mem_bytes = size_t(288) << 30;
+  snprintf(d->props.arch, sizeof(d->props.arch), "gfx950");
+  d->cache_path = cache_dir();
+  *out = d;
+  return WKF_OK;
+}
+
+int wkf_device_is_planner(const wkf_device* dev) { return dev && dev->planner ? 1 : 0; }
+
+int wkf_device_trim(wkf_device* dev) {
+  if (!dev) return fail(WKF_ERR_INVALID_ARG, "wkf_device_trim: null device");
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  if (!dev->planner && dev->pool_bytes) {
+    hipSetDevice(dev->ordinal);
+    hipStreamSynchronize(dev->stream);
+  }
+  for (auto& kv : dev->pool)
+    for (void* p : kv.second) {
+      if (dev->planner) free(p);
+      else hipFree(p);
+    }
+  dev->pool.clear();
+  dev->pool_bytes = 0;
+  return WKF_OK;
+}
+
+void wkf_device_destroy(wkf_device* dev) {
+  if (!dev) return;
+  wkf_device_trim(dev);
+  for (auto& kv : dev->kernels) {
+    if (kv.second->module) hipModuleUnload(kv.second->module);
+    delete kv.second;
+  }
+  if (dev->stream) hipStreamDestroy(dev->stream);
+  delete dev;
+}
+
+int wkf_device_props(wkf_device* dev, wkf_props* out) {
+  if (!dev || !out) return fail(WKF_ERR_INVALID_ARG, "wkf_device_props: null argument");
+  *out = dev->props;
+  return WKF_OK;
+}
+
+int wkf_device_sync(wkf_device* dev) {
+  if (!dev) return fail(WKF_ERR_INVALID_ARG, "wkf_device_sync: null device");
+  if (dev->planner) return WKF_OK;
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  WKF_HIP_CHECK(hipStreamSynchronize(dev->stream));
+  return WKF_OK;
+}
+
+int wkf_buffer_alloc(wkf_device* dev, size_t bytes, int zero_fill, wkf_buffer** out) {
+  if (!dev || !out) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_alloc: null argument");
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  size_t cap = pool_bucket(bytes);
+  void* ptr = nullptr;
+  auto it = dev->pool.find(cap);
+  if (it != dev->pool.end() && !it->second.empty()) {
+    ptr = it->second.back();
+    it->second.pop_back();
+    dev->pool_bytes -= cap;
+  } else if (dev->planner) {
+    ptr = malloc(cap);
+    if (!ptr) return fail(WKF_ERR_OOM, "wkf_buffer_alloc: host allocation failed");
+  } else {
+    WKF_HIP_CHECK(hipSetDevice(dev->ordinal));
+    hipError_t e = hipMalloc(&ptr, cap);
+    if (e == hipErrorOutOfMemory) {
+      // Give cached blocks back to the driver and retry once.
+      (void)hipGetLastError();
+      wkf_device_trim(dev);
+      e = hipMalloc(&ptr, cap);
+    }
+    if (e != hipSuccess)
+      return fail(e == hipErrorOutOfMemory ? WKF_ERR_OOM : WKF_ERR_HIP,
+                  std::string("hipMalloc(") + std::to_string(cap) + "): " + hipGetErrorString(e));
+  }
+  if (zero_fill) {
+    if (dev->planner) memset(ptr, 0, cap);
+    else {
+      hipError_t e = hipMemsetAsync(ptr, 0, cap, dev->stream);
+      if (e != hipSuccess) {
+        hipFree(ptr);
+        return fail(WKF_ERR_HIP, std::string("hipMemsetAsync: ") + hipGetErrorString(e));
+      }
+    }
+  }
+  wkf_buffer* b = new wkf_buffer{dev, ptr, bytes, cap, {1}, false};
+  *out = b;
+  return WKF_OK;
+}
+
+void wkf_buffer_retain(wkf_buffer* buf) {
+  if (buf) buf->refs.fetch_add(1, std::memory_order_relaxed);
+}
+
+void wkf_buffer_release(wkf_buffer* buf) {
+  if (!buf) return;
+  if (buf->refs.fetch_sub(1, std::memory_order_acq_rel) != 1) return;
+  wkf_device* dev = buf->dev;
+  {
+    std::lock_guard<std::recursive_mutex> lock(dev->mu);
+    // Work already queued on the single stream finishes before any later user of
+    // this block starts, so the block can be handed out again without a sync.
+    if (dev->pool_bytes + buf->capacity <= dev->pool_limit) {
+      dev->pool[buf->capacity].push_back(buf->ptr);
+      dev->pool_bytes += buf->capacity;
+    } else if (dev->planner) {
+      free(buf->ptr);
+    } else {
+      hipStreamSynchronize(dev->stream);
+      hipFree(buf->ptr);
+    }
+  }
+  delete buf;
+}
+
+int wkf_buffer_refcount(const wkf_buffer* buf) { return buf ? buf->refs.load(std::memory_order_acquire) : 0; }
+size_t wkf_buffer_size(const wkf_buffer* buf) { return buf ? buf->bytes : 0; }
+void* wkf_buffer_ptr(const wkf_buffer* buf) { return buf ? buf->ptr : nullptr; }
+
+int wkf_buffer_upload(wkf_buffer* buf, size_t offset, const void* src, size_t bytes) {
+  if (!buf || (!src && bytes)) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_upload: null argument");
+  if (offset + bytes > buf->capacity) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_upload: range outside the buffer");
+  if (!bytes) return WKF_OK;
+  wkf_device* dev = buf->dev;
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  if (dev->planner) {
+    memcpy(static_cast<char*>(buf->ptr) + offset, src, bytes);
+    buf->host_valid = true;
+    return WKF_OK;
+  }
+  WKF_HIP_CHECK(hipMemcpyAsync(static_cast<char*>(buf->ptr) + offset, src, bytes, hipMemcpyHostToDevice, dev->stream));
+  // The source is pageable host memory the caller may free on return.
+  WKF_HIP_CHECK(hipStreamSynchronize(dev->stream));
+  return WKF_OK;
+}
+
+int wkf_buffer_download(wkf_buffer* buf, size_t offset, void* dst, size_t bytes) {
+  if (!buf || (!dst && bytes)) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_download: null argument");
+  if (offset + bytes > buf->capacity) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_download: range outside the buffer");
+  if (!bytes) return WKF_OK;
+  wkf_device* dev = buf->dev;
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  if (dev->planner) {
+    if (!buf->host_valid)
+      return fail(WKF_ERR_NO_DEVICE, "wkf_buffer_download: this buffer is the output of a kernel and the device is plan-only (no GPU): nothing was computed");
+    memcpy(dst, static_cast<char*>(buf->ptr) + offset, bytes);
+    return WKF_OK;
+  }
+  WKF_HIP_CHECK(hipMemcpyAsync(dst, static_cast<char*>(buf->ptr) + offset, bytes, hipMemcpyDeviceToHost, dev->stream));
+  WKF_HIP_CHECK(hipStreamSynchronize(dev->stream));
+  return WKF_OK;
+}
+
+int wkf_buffer_copy(wkf_buffer* dst, wkf_buffer* src, size_t bytes) {
+  if (!dst || !src || dst->dev != src->dev) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_copy: bad buffers");
+  if (bytes > dst->capacity || bytes > src->capacity) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_copy: range outside a buffer");
+  wkf_device* dev = dst->dev;
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  if (dev->planner) {
+    memcpy(dst->ptr, src->ptr, bytes);
+    dst->host_valid = src->host_valid;
+    return WKF_OK;
+  }
+  WKF_HIP_CHECK(hipMemcpyAsync(dst->ptr, src->ptr, bytes, hipMemcpyDeviceToDevice, dev->stream));
+  return WKF_OK;
+}
+
+static int load_code(wkf_device* dev, wkf_kernel* k, const std::vector<char>& code) {
+  if (dev->planner) return WKF_OK;  // compiled (or found on disk) but never loaded: no GPU
+  WKF_HIP_CHECK(hipSetDevice(dev->ordinal));
+  WKF_HIP_CHECK(hipModuleLoadData(&k->module, code.data()));
+  WKF_HIP_CHECK(hipModuleGetFunction(&k->function, k->module, k->entry.c_str()));
+  return WKF_OK;
+}
+
+int wkf_module_get(wkf_device* dev, const char* signature, const char* hip_source, const char* entry,
+                   wkf_kernel** out) {
+  if (!dev || !signature || !hip_source || !entry || !out)
+    return fail(WKF_ERR_INVALID_ARG, "wkf_module_get: null argument");
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  auto it = dev->kernels.find(signature);
+  if (it != dev->kernels.end()) {
+    dev->n_mem++;
+    *out = it->second;
+    return WKF_OK;
+  }
+  // Disk key: everything that decides the code object's bytes.
+  uint64_t h = fnv1a(kCacheVersion, strlen(kCacheVersion));
+  for (int i = 0; i < kNumCompileOptions; i++) h = fnv1a(kCompileOptions[i], strlen(kCompileOptions[i]), h);
+  h = fnv1a(entry, strlen(entry), h);
+  h = fnv1a(hip_source, strlen(hip_source), h);
+  char name[64];
+  snprintf(name, sizeof(name), "/%016llx.hsaco", (unsigned long long)h);
+  std::string path = dev->cache_path + name;
+
+  wkf_kernel* k = new wkf_kernel();
+  k->signature = signature;
+  k->entry = entry;
+  std::vector<char> code;
+  bool disk_cache = !(getenv("WKF_NO_DISK_CACHE") && *getenv("WKF_NO_DISK_CACHE") == '1');
+  if (disk_cache) {
+    if (FILE* f = fopen(path.c_str(), "rb")) {
+      fseek(f, 0, SEEK_END);
+      long n = ftell(f);
+      fseek(f, 0, SEEK_SET);
+      if (n > 0) {
+        code.resize(n);
+        if (fread(code.data(), 1, n, f) != size_t(n)) code.clear();
+      }
+      fclose(f);
+    }
+  }
+  if (!code.empty()) {
+    int rc = load_code(dev, k, code);
+    if (rc == WKF_OK) {
+      dev->n_disk++;
+      dev->kernels[signature] = k;
+      *out = k;
+      return WKF_OK;
+    }
+    // A stale or truncated cache entry: fall through to a fresh compile.
+    k->module = nullptr;
+    k->function = nullptr;
+    code.clear();
+  }
+  hiprtcProgram prog;
+  if (hiprtcCreateProgram(&prog, hip_source, "wkf_kernel.hip", 0, nullptr, nullptr) != HIPRTC_SUCCESS) {
+    delete k;
+    return fail(WKF_ERR_HIPRTC, "hiprtcCreateProgram failed");
+  }
+  hiprtcResult r = hiprtcCompileProgram(prog, kNumCompileOptions, const_cast<const char**>(kCompileOptions));
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    delete k;
+    return fail(WKF_ERR_HIPRTC, std::string("hiprtc: ") + hiprtcGetErrorString(r) + " for kernel " + signature + "\n" + log);
+  }
+  size_t n = 0;
+  hiprtcGetCodeSize(prog, &n);
+  code.resize(n);
+  hiprtcGetCode(prog, code.data());
+  hiprtcDestroyProgram(&prog);
+  dev->n_compiled++;
+  if (disk_cache) {
+    std::string tmp = path + "." + std::to_string(getpid()) + ".tmp";
+    if (FILE* f = fopen(tmp.c_str(), "wb")) {
+      bool ok = fwrite(code.data(), 1, code.size(), f) == code.size();
+      fclose(f);
+      if (ok) rename(tmp.c_str(), path.c_str());
+      else unlink(tmp.c_str());
+    }
+  }
+  int rc = load_code(dev, k, code);
+  if (rc != WKF_OK) {
+    delete k;
+    return rc;
+  }
+  dev->kernels[signature] = k;
+  *out = k;
+  return WKF_OK;
+}
+
+int wkf_module_stats(wkf_device* dev, uint64_t* compiled, uint64_t* disk_hits, uint64_t* mem_hits) {
+  if (!dev) return fail(WKF_ERR_INVALID_ARG, "wkf_module_stats: null device");
+  if (compiled) *compiled = dev->n_compiled;
+  if (disk_hits) *disk_hits = dev->n_disk;
+  if (mem_hits) *mem_hits = dev->n_mem;
+  return WKF_OK;
+}
+
+int wkf_launch(wkf_device* dev, wkf_kernel* kernel, const uint32_t grid[3], const uint32_t block[3],
+               uint32_t dyn_lds_bytes, const void* args, size_t arg_bytes, wkf_timer* timer) {
+  if (!dev || !kernel || !grid || !block) return fail(WKF_ERR_INVALID_ARG, "wkf_launch: null argument");
+  uint64_t threads = uint64_t(block[0]) * block[1] * block[2];
+  if (!threads || threads > 1024 || !grid[0] || !grid[1] || !grid[2] || grid[1] > 65535 || grid[2] > 65535)
+    return fail(WKF_ERR_INVALID_ARG, "wkf_launch: bad launch geometry");
+  if (dev->planner) return WKF_OK;  // plan-only: nothing runs
+  if (!kernel->function) return fail(WKF_ERR_INVALID_ARG, "wkf_launch: kernel has no loaded function");
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  size_t size = arg_bytes;
+  void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(args), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
+                    HIP_LAUNCH_PARAM_END};
+  if (timer) WKF_HIP_CHECK(hipEventRecord(timer->begin, dev->stream));
+  WKF_HIP_CHECK(hipModuleLaunchKernel(kernel->function, grid[0], grid[1], grid[2], block[0], block[1], block[2],
+                                      dyn_lds_bytes, dev->stream, nullptr, config));
+  if (timer) {
+    WKF_HIP_CHECK(hipEventRecord(timer->end, dev->stream));
+    timer->recorded = true;
+  }
+  return WKF_OK;
+}
+
+int wkf_timer_create(wkf_device* dev, wkf_timer** out) {
+  if (!dev || !out) return fail(WKF_ERR_INVALID_ARG, "wkf_timer_create: null argument");
+  wkf_timer* t = new wkf_timer();
+  t->dev = dev;
+  if (!dev->planner) {
+    if (hipEventCreate(&t->begin) != hipSuccess || hipEventCreate(&t->end) != hipSuccess) {
+      if (t->begin) hipEventDestroy(t->begin);
+      delete t;
+      return fail(WKF_ERR_HIP, "hipEventCreate failed");
+    }
+  }
+  *out = t;
+  return WKF_OK;
+}
+
+void wkf_timer_destroy(wkf_timer* t) {
+  if (!t) return;
+  if (t->begin) hipEventDestroy(t->begin);
+  if (t->end) hipEventDestroy(t->end);
+  delete t;
+}
+
+int wkf_timer_begin(wkf_timer* t) {
+  if (!t) return fail(WKF_ERR_INVALID_ARG, "wkf_timer_begin: null timer");
+  if (t->dev->planner) return WKF_OK;
+  std::lock_guard<std::recursive_mutex> lock(t->dev->mu);
+  WKF_HIP_CHECK(hipEventRecord(t->begin, t->dev->stream));
+  return WKF_OK;
+}
+
+int wkf_timer_end(wkf_timer* t) {
+  if (!t) return fail(WKF_ERR_INVALID_ARG, "wkf_timer_end: null timer");
+  if (t->dev->planner) return WKF_OK;
+  std::lock_guard<std::recursive_mutex> lock(t->dev->mu);
+  WKF_HIP_CHECK(hipEventRecord(t->end, t->dev->stream));
+  t->recorded = true;
+  return WKF_OK;
+}
+
+int wkf_timer_elapsed_ns(wkf_timer* t, uint64_t* out) {
+  if (!t || !out) return fail(WKF_ERR_INVALID_ARG, "wkf_timer_elapsed_ns: null argument");
+  if (t->dev->planner) {
+    *out = 0;
+    return WKF_OK;
+  }
+  if (!t->recorded) return fail(WKF_ERR_INVALID_ARG, "wkf_timer_elapsed_ns: timer was never recorded");
+  WKF_HIP_CHECK(hipEventSynchronize(t->end));
+  float ms = 0.f;
+  WKF_HIP_CHECK(hipEventElapsedTime(&ms, t->begin, t->end));
+  *out = static_cast<uint64_t>(double(ms) * 1e6);
+  return WKF_OK;
+}
+
+}  // extern "C"
