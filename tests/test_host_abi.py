@@ -1,0 +1,248 @@
+"""Host-side tests that need no GPU: the C ABI loads and exports what the headers
+declare, misuse returns status codes (where the reference panics), layouts are
+decoded on the host, and the fusion pass produces the kernels the reference's
+rules produce.  They run on a plan-only device: kernels are generated and
+JIT-compiled for gfx950 but nothing is launched and nothing is computed."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+
+from helpers import ROOT
+
+
+def _declared_symbols():
+    names = set()
+    for header in ("wkf_hip.h", "wkf_tensor.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(wkf_[a-z0-9_]+)\s*\(", text))
+    return names
+
+
+def test_library_exports_every_declared_symbol(wkf):
+    lib = ctypes.CDLL(wkf.LIB_PATH)
+    declared = _declared_symbols()
+    assert len(declared) > 60
+    missing = [n for n in sorted(declared) if not hasattr(lib, n)]
+    assert not missing, missing
+    assert declared == set(wkf.EXPORTS), declared ^ set(wkf.EXPORTS)
+
+
+def test_headers_cite_the_reference_interface():
+    for header in ("wkf_hip.h", "wkf_tensor.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        assert len(re.findall(r"src/[a-z_/]+\.rs:\d+", text)) >= 15, header
+
+
+def test_planner_device_props(planner):
+    p = planner.props()
+    assert planner.is_planner and p.ordinal == -1 and p.wave_size == 64 and p.arch == b"gfx950"
+
+
+def test_leaf_roundtrip_and_host_side_view_decoding(wkf, planner):
+    data = np.array([[1, 2], [3, 4], [5, 6]], dtype=np.float32)
+    t = wkf.Tensor.new(planner, data)
+    assert t.shape() == (3, 2) and t.rank() == 2 and t.datatype() == wkf.F32
+    assert np.array_equal(t.to_numpy(), data)
+    # test_tensor_slice, src/tensor.rs:646-666 of the reference: the whole buffer comes back, the view is decoded on the host
+    s = t.slice([(0, 2), (0, 1)]).as_slice()
+    assert s.shape == (2, 1) and s.strides == (2, 1) and s.offset == 0 and s.buffer.size == 6
+    assert s[0, 0] == 1.0 and s[1, 0] == 3.0
+    assert s.get([0, 1]) is None and s.get([1, 1]) is None and s.get([2, 0]) is None
+    tr = t.transpose(0, 1).as_slice()
+    assert tr.shape == (2, 3) and tr.strides == (1, 2)
+    assert np.array_equal(tr.to_numpy(), data.T)
+    b = wkf.Tensor.new(planner, np.array([[1, 2], [3, 4]], dtype=np.float32)).broadcast([2, 2, 3]).as_slice()
+    assert b.shape == (2, 2, 3) and b.strides == (2, 1, 0)
+    n = t.narrow(0, 1, 2).as_slice()
+    assert n.offset == 2 and np.array_equal(n.to_numpy(), data[1:])
+    # test_tensor_compare, src/tensor.rs:786-815
+    cube = wkf.Tensor.new(planner, np.arange(24, dtype=np.float32).reshape(6, 2, 2))
+    a = cube.slice([(0, 2), (0, 1), (0, 1)]).as_slice()
+    assert a == a
+    assert a != cube.slice([(0, 1), (0, 1), (0, 1)]).as_slice()
+    assert a != cube.slice([(1, 3), (0, 1), (0, 1)]).as_slice()
+    h = wkf.Tensor.new(planner, data.astype(np.float16))
+    assert h.datatype() == wkf.F16 and np.array_equal(h.to_numpy(), data.astype(np.float16))
+
+
+def test_computed_values_are_refused_without_a_gpu(wkf, planner):
+    t = wkf.Tensor.new(planner, np.ones((4, 4), dtype=np.float32)) + 1.0
+    t.materialize()  # planning and compiling is fine
+    with pytest.raises(wkf.WkfError) as e:
+        t.as_slice()
+    assert e.value.code == 5 and "plan-only" in str(e.value)
+
+
+def test_misuse_returns_status_codes(wkf, planner):
+    T = wkf.Tensor
+    a = T.new(planner, np.ones((3, 2), dtype=np.float32))
+    b = T.new(planner, np.ones((2, 3), dtype=np.float32))
+    h = T.new(planner, np.ones((3, 2), dtype=np.float16))
+    cases = [
+        lambda: a + b,                       # src/pair_wise.rs:92
+        lambda: a + h,                       # dtype mismatch (a compile error in Rust)
+        lambda: a.sum(2),                    # axis out of range
+        lambda: a.mat_mul(a),                # src/matmul.rs:194
+        lambda: a.narrow(0, 2, 2),           # src/composite/narrow.rs:6
+        lambda: a.narrow(2, 0, 1),           # src/composite/narrow.rs:7
+        lambda: a.broadcast([3, 2]),         # rank must grow by one
+        lambda: a.broadcast([3, 5, 7]),      # src/map_layout.rs:78-79
+        lambda: a.reshape([4, 2]),           # src/resize.rs:132-135
+        lambda: a.slice([(0, 4), (0, 2)]),   # range outside the tensor
+        lambda: a.slice_assign([(0, 2), (0, 2)], b),  # src/slice_assign.rs:69
+        lambda: T.cat([a, b], 0),            # src/composite/cat.rs:12-19
+        lambda: T.cat([a, a], 2),
+        lambda: a.softmax(),                 # rank 1 only
+        lambda: a.layer_norm(T.new(planner, np.ones(3, dtype=np.float32)), 1e-5),
+        lambda: T.arange_step(planner, 0.0, 1.0, 0.0),
+    ]
+    for i, f in enumerate(cases):
+        with pytest.raises(wkf.WkfError) as e:
+            f()
+        assert e.value.code == 3, (i, str(e.value))
+    with pytest.raises(ValueError):
+        T.new(planner, [[1.0, 2.0], [3.0]])  # ragged input: the reference panics in IntoTensor
+    with pytest.raises(wkf.WkfError):
+        wkf.Device.new(99)
+
+
+def test_hiprtc_failure_is_reported_with_the_log(wkf, planner):
+    lib = wkf.load()
+    k = ctypes.c_void_p()
+    rc = lib.wkf_module_get(planner._h, b"test|bad-source", b"extern \"C\" __global__ void k() { this is not HIP }", b"k",
+                            ctypes.byref(k))
+    assert rc == 2
+    msg = lib.wkf_last_error().decode()
+    assert "hiprtc" in msg and "error" in msg
+
+
+def test_arange_is_a_host_loop(wkf, planner):
+    assert np.array_equal(wkf.Tensor.arange(planner, 0.0, 10.0).to_numpy(), np.arange(10, dtype=np.float32))
+    assert np.array_equal(wkf.Tensor.arange_step(planner, 0.0, 10.0, 2.0).to_numpy(), np.array([0, 2, 4, 6, 8], dtype=np.float32))
+    assert np.array_equal(wkf.Tensor.arange_step(planner, 3.0, 0.0, -1.0).to_numpy(), np.array([3, 2, 1], dtype=np.float32))
+    h = wkf.Tensor.arange_step(planner, 0.0, 1.0, 0.25, dtype=wkf.F16)
+    assert h.datatype() == wkf.F16 and np.array_equal(h.to_numpy(), np.array([0, 0.25, 0.5, 0.75], dtype=np.float16))
+
+
+# ---- the fusion pass (src/compute_graph/resolve.rs:49-196 of the reference) ---------------------
+
+def _kinds(t):
+    t.materialize()
+    return [k.kind for k in t.kernels()]
+
+
+def _x(wkf, dev, shape=(64, 64), dtype=np.float32, seed=0):
+    return wkf.Tensor.new(dev, np.random.default_rng(seed).standard_normal(shape).astype(dtype))
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_fusion_rules_shared_by_both_modes(wkf, planner, mode):
+    planner.set_fusion(mode)
+    try:
+        x, y = _x(wkf, planner), _x(wkf, planner, seed=1)
+        # (1) a chain of element-wise nodes is one kernel (test_merge_add_const, src/element_wise.rs:422-443)
+        t = ((x * 2.0) + 1.0).sin().exp()
+        assert _kinds(t) == ["map"]
+        sig = t.kernels()[0].signature
+        assert "multiply_const" in sig and "add_const" in sig and "sin" in sig and "exp" in sig
+        assert not t.kernels()[0].detail.endswith("in_place")  # a leaf is never overwritten (tests/inplace_clone.rs)
+        # (3) chains below both operands of a pair-wise op fuse into it (src/pair_wise.rs:292-317)
+        assert _kinds((x + 1.0) + (y * 2.0)) == ["map"]
+        # (2) a chain above a pair-wise op fuses into it (src/pair_wise.rs:321-346)
+        assert _kinds((x + y) - 1.0) == ["map"]
+        # (3) pre-fused reduce (src/reduce.rs:570-600) and (2) post-fused reduce (:604-631)
+        assert _kinds((x + 1.0).sum(0)) == ["red_col"]
+        assert _kinds((x + 1.0).sum(1)) == ["red_row"]
+        r = x.sum(1) + 1.0
+        assert _kinds(r) == ["red_row"] and "post:load:f32@0;add_const" in r.kernels()[0].signature
+        # (4) views cost nothing; a reduce of a sliced view still is one kernel
+        assert _kinds(x.slice([(0, 64), (0, 1)]).sum(0)) == ["red_col"]
+        assert _kinds(x.transpose(0, 1)) == []
+        # (5) reduce <-> reduce never fuse
+        assert _kinds(x.sum(1).sum(0)) == ["red_row", "red_row"]
+        # resize, slice_assign and cat are copies
+        assert _kinds(x.resize([70, 80])) == ["map"]
+        assert _kinds(x.reshape([32, 128])) == ["map"]
+    finally:
+        planner.set_fusion(1)
+
+
+def test_reference_mode_is_the_reference_decomposition(wkf, planner):
+    planner.set_fusion(wkf.FUSION_REFERENCE)
+    try:
+        a, b = _x(wkf, planner, (4, 8, 16)), _x(wkf, planner, (4, 8, 16), seed=1)
+        bias = _x(wkf, planner, (16,), seed=2)
+        bias3 = bias.broadcast([8, 16]).broadcast([4, 8, 16])
+        out = a.silu() * (b + bias3)
+        # silu's div, the strided add, then the mul in place into the div's result (src/pair_wise.rs:95-107)
+        assert _kinds(out) == ["map", "map", "map"]
+        ks = out.kernels()
+        assert "in_place" not in ks[0].detail and "in_place" not in ks[1].detail and ks[2].detail.endswith("in_place")
+        # RMSNorm = one reduce (pre [sqr], post [/H, +eps, sqrt]) + two strided pair-wise kernels
+        x, w = _x(wkf, planner, (32, 64)), _x(wkf, planner, (64,), seed=3)
+        ln = x.layer_norm(w, 1e-5)
+        assert _kinds(ln) == ["red_row", "map", "map"]
+        sig = ln.kernels()[0].signature
+        assert "pre:load:f32@0;sqr" in sig and "divide_const" in sig and "add_const" in sig and "sqrt" in sig
+        # no memoisation: the exp under softmax is computed in both kernels (src/tensor.rs:286-288)
+        v = _x(wkf, planner, (128,))
+        assert _kinds(v.softmax()) == ["red_row", "map"]
+        # (5) pair-wise <-> pair-wise do not fuse: (a + b) is materialised, then multiplied in place
+        t = (a + b) * a
+        assert _kinds(t) == ["map", "map"] and t.kernels()[1].detail.endswith("in_place")
+    finally:
+        planner.set_fusion(wkf.FUSION_TREE)
+
+
+def test_tree_mode_fuses_pair_wise_trees_and_copies(wkf, planner):
+    a, b = _x(wkf, planner, (4, 8, 16)), _x(wkf, planner, (4, 8, 16), seed=1)
+    bias3 = _x(wkf, planner, (16,), seed=2).broadcast([8, 16]).broadcast([4, 8, 16])
+    out = a.silu() * (b + bias3)
+    assert _kinds(out) == ["map"]
+    k = out.kernels()[0]
+    assert "operands=4" in k.detail  # a (read once although silu uses it twice), b, bias, out
+    assert "shape=[32,16]" in k.detail  # the two leading dims merge for every operand
+    x, w = _x(wkf, planner, (32, 64)), _x(wkf, planner, (64,), seed=3)
+    assert _kinds(x.layer_norm(w, 1e-5)) == ["red_row", "map"]
+    s = _x(wkf, planner, (4, 8, 32)).softmax_last_dim()
+    assert _kinds(s) == ["red_row", "red_row", "map"]  # max once (shared), sum(exp(x - max)), exp(x - max) / sum
+    q = _x(wkf, planner, (2, 8, 16))
+    cos, sin = _x(wkf, planner, (8, 8), seed=4), _x(wkf, planner, (8, 8), seed=5)
+    kinds = _kinds(q.rope(cos, sin))
+    assert all(k == "map" for k in kinds) and len(kinds) <= 8
+
+
+def test_one_binary_serves_every_size_and_constant(wkf, planner):
+    before = planner.module_stats()
+    t1 = (_x(wkf, planner, (256, 256)) * 3.0) + 5.0
+    t2 = (_x(wkf, planner, (128, 512)) * -7.5) + 0.25
+    t1.materialize()
+    t2.materialize()
+    assert t1.kernels()[0].signature == t2.kernels()[0].signature
+    after = planner.module_stats()
+    assert after["compiled"] + after["disk_hits"] - before["compiled"] - before["disk_hits"] <= 1
+    assert after["mem_hits"] >= before["mem_hits"] + 1
+
+
+def test_generated_source_keeps_every_op_rounded_on_its_own(wkf, planner):
+    t = ((_x(wkf, planner, (64, 64), np.float16) * 2.0) + 1.0).exp()
+    t.materialize()
+    src = wkf.kernel_source(t.kernels()[0].signature)
+    assert "const _Float16 v1 = v0 * (_Float16)c[0];" in src
+    assert "const _Float16 v2 = v1 + (_Float16)c[1];" in src
+    assert "wkf_f16x8" in src  # 128-bit vectors of f16
+    f = ((_x(wkf, planner, (64, 64)) * 2.0) + 1.0).sin().exp()
+    f.materialize()
+    src = wkf.kernel_source(f.kernels()[0].signature)
+    assert "wkf_sin(v2, far)" in src and "expf(v3)" in src  # interior op: f64 core; last op: f32 library
+    assert "wkf_expr_far" in src and "wkf_f32x4" in src
+    planner.set_exact_math(True)
+    try:
+        f.materialize()
+        assert "wkf_exp(v3)" in wkf.kernel_source(f.kernels()[0].signature)
+    finally:
+        planner.set_exact_math(False)

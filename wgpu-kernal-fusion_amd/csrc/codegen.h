@@ -104,19 +104,12 @@ struct ReduceArgs {
 std::vector<unsigned char> reduce_pack_args(const ReduceSpec& s, const ReduceArgs& a);
 
 // ---- GEMM ----------------------------------------------------------------------
-// K4 of the reference (src/matmul.rs:56-155) re-designed for MFMA.
-struct GemmSpec {
-  DType dtype;       // A, B and C share it (src/matmul.rs:157-183)
-  int tile_m, tile_n, tile_k;
-  int waves_m, waves_n;
-  bool exact_tiles;  // M, N, K are multiples of the tile: no edge handling
-};
-std::string gemm_signature(const GemmSpec& s);
-std::string gemm_source(const GemmSpec& s);
-struct GemmArgs {
-  const void* a; const void* b; void* c;
-  uint32_t m, n, k;
-};
-std::vector<unsigned char> gemm_pack_args(const GemmArgs& a);
+// K4 of the reference (src/matmul.rs:56-155) re-designed for MFMA: hand-written
+// kernels (kernels/gemm_*.hip.inc), chosen by dtype and by whether the shape is
+// a multiple of the 256 x 256 x BK tile.
+enum class GemmKind { MfmaF16, MfmaF32, Generic };
+GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k);
+std::string gemm_signature(GemmKind kind, DType dt);
+std::string gemm_source(GemmKind kind, DType dt);
 
 }  // namespace wkf

@@ -203,16 +203,22 @@ TensorData Resolver::resolve_root(const NodeP& root) {
   std::set<const Node*>& shared = shared_;
   shared.clear();
   materialized_.clear();
+  // An element-wise or pair-wise node is inlined into every kernel that uses it,
+  // so its second use is also a second use of its inputs: the walk goes through
+  // it twice.  Any other node is cut off at its second use.
   std::function<void(const NodeP&)> walk = [&](const NodeP& n) {
     if (!n) return;
-    if (++uses[n.get()] > 1) {
+    const int seen = ++uses[n.get()];
+    if (seen > 2) return;
+    if (seen == 2) {
       shared.insert(n.get());
-      return;
+      if (n->kind != NodeKind::ElementWise && n->kind != NodeKind::PairWise) return;
     }
     walk(n->a);
     walk(n->b);
   };
-  walk(root);
+  // Under the reference rules nothing is shared: a node used twice is computed twice.
+  if (st_.fusion == FusionMode::Tree) walk(root);
   shared.erase(root.get());
   TensorData out = resolve(root);
   materialized_.clear();
