@@ -69,6 +69,11 @@ int wkf_device_get_fusion(wkf_device* dev);
  * exact != 0: every transcendental op is evaluated in f64 and rounded once. */
 int wkf_device_set_exact_math(wkf_device* dev, int exact);
 
+/* Per-kernel GPU timestamps (PerformanceQueries, src/query.rs:50-126: the reference
+ * attaches one to every kernel).  On by default; a caller that only wants results can
+ * switch the hipEvent pair per launch off. */
+int wkf_device_set_timing(wkf_device* dev, int enabled);
+
 /* Tensor::new, src/tensor.rs:518-531 (+ IntoTensor :441-515): uploads `data`
  * (row-major, numel * sizeof(dtype) bytes) into a new leaf tensor. */
 int wkf_tensor_new(wkf_device* dev, int dtype, int rank, const size_t* shape, const void* data, wkf_tensor** out);

@@ -281,7 +281,7 @@ std::string map_source(const MapSpec& s) {
     for (int j = j0; j < j1; j++) emit_store(j, ind.c_str());
   };
 
-  o << "extern \"C\" __global__ void __launch_bounds__(" << kMapBlock << ") wkf_kernel(const Args a) {\n";
+  o << "extern \"C\" __global__ void __launch_bounds__(" << kMapBlock << ") WKF_ENTRY(const Args a) {\n";
   o << "  const u32 w_block = blockIdx.x * " << kMapBlock * U << "u;\n";
   o << "  const u32 w_first = w_block + threadIdx.x;\n";
   o << "  if (w_block + " << kMapBlock * U << "u <= a.nwork) {\n";
@@ -394,7 +394,7 @@ std::string reduce_source(const ReduceSpec& s) {
   if (s.shape == ReduceShape::Row) {
     const int T = s.threads_per_row, V = s.vec, U = s.unroll, B = s.block;
     const int RPB = B / T;
-    o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") wkf_kernel(const Args a) {\n";
+    o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") WKF_ENTRY(const Args a) {\n";
     if (T > 64) o << "  __shared__ float wkf_partial[" << B / 64 << "];\n";
     o << "  const u32 t = threadIdx.x % " << T << "u;\n";
     o << "  const u32 row_raw = blockIdx.x * " << RPB << "u + threadIdx.x / " << T << "u;\n";
@@ -467,7 +467,7 @@ std::string reduce_source(const ReduceSpec& s) {
     o << "}\n";
   } else {
     const int W = s.waves;
-    o << "extern \"C\" __global__ void __launch_bounds__(" << 64 * W << ") wkf_kernel(const Args a) {\n";
+    o << "extern \"C\" __global__ void __launch_bounds__(" << 64 * W << ") WKF_ENTRY(const Args a) {\n";
     if (W > 1) o << "  __shared__ float wkf_partial[" << W << "][64];\n";
     o << "  const u32 lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;\n";
     // The 64 lanes of a wave sit on 64 neighbouring positions of the LAST outer dim.

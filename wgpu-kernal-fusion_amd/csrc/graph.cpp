@@ -137,13 +137,29 @@ TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero
 extern std::mutex g_source_mu;
 extern std::unordered_map<std::string, std::string> g_sources;
 
-wkf_kernel* Resolver::kernel(const std::string& sig, const std::string& src) {
+// Every kernel gets its own entry-point name, "wkf_<kind>_<hash of the signature>", so that
+// profilers list fused kernels separately.
+static std::string entry_name(const std::string& sig) {
+  uint64_t h = 1469598103934665603ull;
+  for (unsigned char c : sig) {
+    h ^= c;
+    h *= 1099511628211ull;
+  }
+  char buf[80];
+  std::string kind = sig.substr(0, sig.find('|'));
+  snprintf(buf, sizeof(buf), "wkf_%s_%08x", kind.c_str(), unsigned(h ^ (h >> 32)));
+  return buf;
+}
+
+wkf_kernel* Resolver::kernel(const std::string& sig, const std::string& body) {
+  const std::string entry = entry_name(sig);
+  const std::string src = "#define WKF_ENTRY " + entry + "\n" + body;
   {
     std::lock_guard<std::mutex> lock(g_source_mu);
     g_sources.emplace(sig, src);
   }
   wkf_kernel* k = nullptr;
-  check(wkf_module_get(dev_, sig.c_str(), src.c_str(), "wkf_kernel", &k));
+  check(wkf_module_get(dev_, sig.c_str(), src.c_str(), entry.c_str(), &k));
   return k;
 }
 

@@ -396,6 +396,14 @@ int wkf_device_set_fusion(wkf_device* dev, int mode) {
 
 int wkf_device_get_fusion(wkf_device* dev) { return int(settings_for(dev).fusion); }
 
+int wkf_device_set_timing(wkf_device* dev, int enabled) {
+  return guarded([&] {
+    need(dev, "wkf_device_set_timing");
+    std::lock_guard<std::mutex> lock(g_settings_mu);
+    g_settings[dev].timing = enabled != 0;
+  });
+}
+
 int wkf_device_set_exact_math(wkf_device* dev, int exact) {
   return guarded([&] {
     need(dev, "wkf_device_set_exact_math");
