@@ -88,6 +88,11 @@ int wkf_buffer_copy(wkf_buffer* dst, wkf_buffer* src, size_t bytes);
  * hipModuleGetFunction).  The returned kernel is owned by the device. */
 int wkf_module_get(wkf_device* dev, const char* signature, const char* hip_source,
                    const char* entry, wkf_kernel** out);
+/* Memory-cache lookup only: *out is the kernel, or NULL when this device has not seen the
+ * signature yet (the caller then generates the source and calls wkf_module_get).  Lets the
+ * generator skip building source text on the hot path; no reference counterpart (the reference
+ * regenerates and recompiles its WGSL on every launch, src/kernel.rs:262-271,371-373). */
+int wkf_module_find(wkf_device* dev, const char* signature, wkf_kernel** out);
 /* Cache statistics since device creation: kernels compiled by hiprtc, loaded
  * from disk, and served from memory. */
 int wkf_module_stats(wkf_device* dev, uint64_t* compiled, uint64_t* disk_hits, uint64_t* mem_hits);

@@ -207,9 +207,13 @@ def test_tree_mode_fuses_pair_wise_trees_and_copies(wkf, planner):
     assert "operands=4" in k.detail  # a (read once although silu uses it twice), b, bias, out
     assert "shape=[32,16]" in k.detail  # the two leading dims merge for every operand
     x, w = _x(wkf, planner, (32, 64)), _x(wkf, planner, (64,), seed=3)
-    assert _kinds(x.layer_norm(w, 1e-5)) == ["red_row", "map"]
+    # last-axis reductions that are used again on the same rows run as ONE row kernel (row held in registers)
+    ln = x.layer_norm(w, 1e-5)
+    assert _kinds(ln) == ["row"] and "stages=1" in ln.kernels()[0].detail
     s = _x(wkf, planner, (4, 8, 32)).softmax_last_dim()
-    assert _kinds(s) == ["red_row", "red_row", "map"]  # max once (shared), sum(exp(x - max)), exp(x - max) / sum
+    assert _kinds(s) == ["row"] and "stages=2" in s.kernels()[0].detail  # max, sum(exp(x - max)), exp(x - max) / sum
+    # a row length the row kernel does not take (not a multiple of the vector width) falls back to separate kernels
+    assert _kinds(_x(wkf, planner, (8, 30)).softmax_last_dim()) == ["red_row", "red_row", "map"]
     q = _x(wkf, planner, (2, 8, 16))
     cos, sin = _x(wkf, planner, (8, 8), seed=4), _x(wkf, planner, (8, 8), seed=5)
     kinds = _kinds(q.rope(cos, sin))

@@ -36,7 +36,7 @@ EXPORTS = [
     "wkf_device_create", "wkf_device_create_planner", "wkf_device_destroy", "wkf_device_is_planner",
     "wkf_device_props", "wkf_device_sync", "wkf_device_trim", "wkf_buffer_alloc", "wkf_buffer_retain",
     "wkf_buffer_release", "wkf_buffer_refcount", "wkf_buffer_size", "wkf_buffer_ptr", "wkf_buffer_upload",
-    "wkf_buffer_download", "wkf_buffer_copy", "wkf_module_get", "wkf_module_stats", "wkf_launch",
+    "wkf_buffer_download", "wkf_buffer_copy", "wkf_module_get", "wkf_module_find", "wkf_module_stats", "wkf_launch",
     "wkf_timer_create", "wkf_timer_destroy", "wkf_timer_begin", "wkf_timer_end", "wkf_timer_elapsed_ns",
     "wkf_last_error",
     "wkf_device_set_fusion", "wkf_device_get_fusion", "wkf_device_set_exact_math", "wkf_device_set_timing", "wkf_tensor_new", "wkf_tensor_clone", "wkf_tensor_free",

@@ -537,3 +537,183 @@ std::vector<unsigned char> reduce_pack_args(const ReduceSpec& s, const ReduceArg
 }
 
 }  // namespace wkf
+
+// ===========================================================================
+// row kernels
+// ===========================================================================
+namespace wkf {
+namespace {
+const char* const kRowHelpers =
+#include "kernels/row_helpers.hip.inc"
+    ;
+const char* fold_text(ReduceOp r) {
+  switch (r) {
+    case ReduceOp::Sum: return "v + a";
+    case ReduceOp::Max: return "fmaxf(v, a)";
+    case ReduceOp::Min: return "fminf(v, a)";
+    case ReduceOp::Product: return "v * a";
+  }
+  return "";
+}
+const char* seed_text(ReduceOp r) {
+  switch (r) {
+    case ReduceOp::Sum: return "0.0f";
+    case ReduceOp::Max: return "-3.40282e+38f";
+    case ReduceOp::Min: return "3.40282e+38f";
+    case ReduceOp::Product: return "1.0f";
+  }
+  return "";
+}
+}  // namespace
+
+std::string row_signature(const RowSpec& s) {
+  std::ostringstream o;
+  o << "row|gfx950|or" << s.outer_rank << "|v" << s.vec << "|t" << s.threads_per_row << "|b" << s.block << "|nv"
+    << s.vectors_per_lane << "|x" << int(s.exact_math) << "|in:";
+  for (const auto& i : s.in) o << dtype_name(i.dtype) << 'a' << i.axis_stride << ',';
+  o << "|out:" << dtype_name(s.out_dtype);
+  for (const auto& st : s.stages) o << "|" << reduce_name(st.rop) << "{" << st.pre.signature() << "}{" << st.post.signature() << "}";
+  o << "|final{" << s.final.signature() << "}";
+  return o.str();
+}
+
+std::string row_source(const RowSpec& s) {
+  const int K = int(s.in.size()), S = int(s.stages.size());
+  const int Ro = s.outer_rank, T = s.threads_per_row, V = s.vec, NV = s.vectors_per_lane, B = s.block;
+  const int RPB = B / T;
+  const MathPolicy fold_policy = s.exact_math ? MathPolicy::Exact : MathPolicy::Folded;
+  // Everything a row kernel stores is combined with a fold result, so it is in the reduction
+  // tolerance class (1e-5 relative) as a whole: the f32 library is used throughout.
+  const MathPolicy store_policy = fold_policy;
+  int nc = 0;
+  std::vector<int> pre_off, post_off;
+  for (const auto& st : s.stages) {
+    pre_off.push_back(nc);
+    nc += int(st.pre.consts.size());
+    post_off.push_back(nc);
+    nc += int(st.post.consts.size());
+  }
+  const int final_off = nc;
+  nc += int(s.final.consts.size());
+  std::ostringstream o;
+  o << kPrelude;
+  bool math = uses_math(s.final, store_policy);
+  for (const auto& st : s.stages) math |= uses_math(st.pre, fold_policy) || uses_math(st.post, store_policy);
+  if (math) o << kMath;
+  o << kRowHelpers;
+  o << "struct Args { void* p[" << K + 1 << "]; u32 nrows; u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + 1
+    << "]; u32 ostride[" << K + 1 << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
+  // operand types as every program sees them: the K full operands, then one scalar per earlier stage
+  std::vector<DType> types;
+  for (const auto& i : s.in) types.push_back(i.dtype);
+  for (int k = 0; k < S; k++) {
+    std::vector<DType> tk = types;
+    emit_program(o, s.stages[k].pre, "wkf_pre" + std::to_string(k), tk, fold_policy);
+    emit_program(o, s.stages[k].post, "wkf_post" + std::to_string(k), {s.stages[k].pre.result_dtype()}, store_policy);
+    types.push_back(s.stages[k].post.result_dtype());
+  }
+  emit_program(o, s.final, "wkf_final", types, store_policy);
+
+  o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") WKF_ENTRY(const Args a) {\n";
+  if (T > 64) o << "  __shared__ float wkf_partial[" << std::max(1, S) << "][" << B / 64 << "];\n";
+  o << "  const u32 t = threadIdx.x % " << T << "u;\n";
+  o << "  const u32 row_raw = blockIdx.x * " << RPB << "u + threadIdx.x / " << T << "u;\n";
+  o << "  const bool live = row_raw < a.nrows;\n";
+  o << "  const u32 row = live ? row_raw : 0u;\n";
+  if (Ro > 0) {
+    o << "  u32 rem = row;\n";
+    for (int d = Ro - 1; d > 0; d--) o << "  const u32 i" << d << " = rem % a.oshape[" << d << "]; rem /= a.oshape[" << d << "];\n";
+    o << "  const u32 i0 = rem;\n";
+  }
+  auto base_expr = [&](int k) {
+    std::ostringstream e;
+    e << "a.off[" << k << "]";
+    for (int d = 0; d < Ro; d++) e << " + i" << d << " * a.ostride[" << k << "][" << d << "]";
+    return e.str();
+  };
+  // the row of every operand comes into registers once
+  for (int k = 0; k < K; k++) {
+    const char* ct = ctype(s.in[k].dtype);
+    o << "  const " << ct << "* q" << k << " = ((const " << ct << "*)a.p[" << k << "]) + (" << base_expr(k) << ");\n";
+    if (s.in[k].axis_stride == 0) {
+      o << "  const " << ct << " s" << k << " = q" << k << "[0];\n";
+    } else {
+      std::string vt = vtype(s.in[k].dtype, V);
+      for (int j = 0; j < NV; j++)
+        o << "  const " << vt << " x" << k << "_" << j << " = __builtin_nontemporal_load((const " << vt << "*)(q" << k << " + (t + "
+          << j * T << "u) * " << V << "u));\n";
+    }
+  }
+  auto call_args = [&](int j, int e, int nscalars) {
+    std::ostringstream c;
+    for (int k = 0; k < K; k++) {
+      if (s.in[k].axis_stride == 0) c << "s" << k;
+      else {
+        c << "x" << k << "_" << j;
+        if (V > 1) c << "[" << e << "]";
+      }
+      c << ", ";
+    }
+    for (int q = 0; q < nscalars; q++) c << "r" << q << ", ";
+    return c.str();
+  };
+  for (int k = 0; k < S; k++) {
+    const RowStage& st = s.stages[k];
+    o << "  float acc" << k << " = " << seed_text(st.rop) << ";\n";
+    o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(st.rop) << "; };\n";
+    for (int j = 0; j < NV; j++)
+      for (int e = 0; e < V; e++)
+        o << "  acc" << k << " = fold" << k << "((float)wkf_pre" << k << "(" << call_args(j, e, k) << "a.c + " << pre_off[k] << "), acc"
+          << k << ");\n";
+    if (T > 1) o << "  acc" << k << " = wkf_lanes_fold_with<" << std::min(T, 64) << ">(acc" << k << ", fold" << k << ");\n";
+    if (T > 64) {
+      const int WPR = T / 64;
+      o << "  if ((threadIdx.x & 63u) == 0u) wkf_partial[" << k << "][threadIdx.x >> 6] = acc" << k << ";\n";
+      o << "  __syncthreads();\n";
+      o << "  {\n    const u32 first_wave = (threadIdx.x / " << T << "u) * " << WPR << "u;\n";
+      o << "    acc" << k << " = wkf_partial[" << k << "][first_wave];\n";
+      o << "    for (u32 w = 1; w < " << WPR << "u; w++) acc" << k << " = fold" << k << "(wkf_partial[" << k << "][first_wave + w], acc" << k
+        << ");\n  }\n";
+    }
+    o << "  const " << ctype(st.post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(st.pre.result_dtype()) << ")acc" << k
+      << ", a.c + " << post_off[k] << ");\n";
+  }
+  const char* ot = ctype(s.out_dtype);
+  o << "  if (live) {\n";
+  o << "    " << ot << "* qo = ((" << ot << "*)a.p[" << K << "]) + (" << base_expr(K) << ");\n";
+  for (int j = 0; j < NV; j++) {
+    std::string vt = vtype(s.out_dtype, V);
+    o << "    " << vt << " o" << j << ";\n";
+    for (int e = 0; e < V; e++) {
+      o << "    o" << j;
+      if (V > 1) o << "[" << e << "]";
+      o << " = wkf_final(" << call_args(j, e, S) << "a.c + " << final_off << ");\n";
+    }
+    o << "    __builtin_nontemporal_store(o" << j << ", (" << vt << "*)(qo + (t + " << j * T << "u) * " << V << "u));\n";
+  }
+  o << "  }\n}\n";
+  return o.str();
+}
+
+std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a) {
+  const size_t K = s.in.size(), Ro = size_t(s.outer_rank);
+  if (a.ptrs.size() != K + 1 || a.oshape.size() != Ro || a.offsets.size() != K + 1 || a.ostrides.size() != K + 1)
+    throw Error(WKF_ERR_INVALID_ARG, "row_pack_args: argument arity does not match the kernel");
+  std::vector<unsigned char> b;
+  for (void* p : a.ptrs) putp(b, p);
+  put32(b, a.nrows);
+  for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? a.oshape[d] : 1);
+  for (uint32_t v : a.offsets) put32(b, v);
+  for (const auto& st : a.ostrides) {
+    if (st.size() != Ro) throw Error(WKF_ERR_INVALID_ARG, "row_pack_args: stride rank mismatch");
+    for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? st[d] : 0);
+  }
+  size_t nc = s.final.consts.size();
+  for (const auto& st : s.stages) nc += st.pre.consts.size() + st.post.consts.size();
+  nc = std::max<size_t>(1, nc);
+  for (size_t i = 0; i < nc; i++) putf(b, i < a.consts.size() ? a.consts[i] : 0.f);
+  pad8(b);
+  return b;
+}
+
+}  // namespace wkf

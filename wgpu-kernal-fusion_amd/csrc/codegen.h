@@ -103,6 +103,43 @@ struct ReduceArgs {
 };
 std::vector<unsigned char> reduce_pack_args(const ReduceSpec& s, const ReduceArgs& a);
 
+// ---- row kernels: reductions over the last axis whose results are used again on the same rows ----
+// softmax (max -> sum(exp(x - max)) -> exp(x - max) / sum) and RMSNorm (sum(x^2) -> x / rms * w) read
+// each row once: T lanes hold the row of every operand in registers, each `stage` folds an
+// expression over the row into one scalar per row (which later stages and the final expression may
+// use), and the final expression is stored.  No counterpart in the reference, which runs one kernel
+// per reduce and per pair-wise op (src/compute_graph/resolve.rs:96-196); the values are the same.
+struct RowStage {
+  ReduceOp rop;
+  Program pre;    // operands: full operands 0..K-1, then the scalars of earlier stages K..K+s-1
+  Program post;   // one Load (operand 0 = the folded value)
+};
+
+struct RowSpec {
+  int outer_rank;                       // dims of the row index space (coalesced), 0..3
+  int vec;                              // elements per 16-byte load
+  int threads_per_row;                  // T
+  int block;                            // threads per block
+  int vectors_per_lane;                 // NV: row length = NV * T * vec exactly
+  std::vector<ReduceOperandSpec> in;    // axis_stride 1 (row in registers) or 0 (one scalar per row)
+  std::vector<RowStage> stages;
+  Program final;                        // same operand numbering as a stage's pre
+  DType out_dtype;
+  bool exact_math = false;
+};
+
+std::string row_signature(const RowSpec& s);
+std::string row_source(const RowSpec& s);
+struct RowArgs {
+  std::vector<void*> ptrs;                        // inputs..., out
+  uint32_t nrows;
+  std::vector<uint32_t> oshape;
+  std::vector<uint32_t> offsets;                  // per operand incl. out
+  std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. out, per outer dim
+  std::vector<float> consts;                      // stage 0 pre, stage 0 post, stage 1 pre, ..., final
+};
+std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a);
+
 // ---- GEMM ----------------------------------------------------------------------
 // K4 of the reference (src/matmul.rs:56-155) re-designed for MFMA: hand-written
 // kernels (kernels/gemm_*.hip.inc), chosen by dtype and by whether the shape is

@@ -62,7 +62,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
 
   const GemmKind kind = gemm_pick(a.dtype, M, N, K);
   std::string sig = gemm_signature(kind, a.dtype);
-  wkf_kernel* k = kernel(sig, gemm_source(kind, a.dtype));
+  wkf_kernel* k = kernel(sig, [&] { return gemm_source(kind, a.dtype); });
 
   struct {
     const void* a;

@@ -106,7 +106,12 @@ int Resolver::build(ExprBuilder& eb, const NodeP& n, int pairwise_budget) {
   int v;
   // Keep kernels within a sane register / argument budget: past it, a sub-tree is materialised.
   const bool room = eb.prog.ins.size() < 48 && eb.operands.size() < 7;
-  if (n->kind == NodeKind::ElementWise) {
+  if (eb.split && n.get() == eb.split->cat) {
+    const bool was = eb.inside_piece;
+    eb.inside_piece = true;  // operands below are already piece-shaped
+    v = build(eb, eb.split->piece, pairwise_budget);
+    eb.inside_piece = was;
+  } else if (n->kind == NodeKind::ElementWise) {
     int a = build(eb, n->a, pairwise_budget);
     v = eb.emit(n->op, a, -1, n->dtype, is_const_op(n->op), n->constant);
   } else if (n->kind == NodeKind::PairWise && pairwise_budget > 0 && room) {
@@ -115,11 +120,55 @@ int Resolver::build(ExprBuilder& eb, const NodeP& n, int pairwise_budget) {
     v = eb.emit(n->op, a, b, n->dtype, false, 0.f);
   } else {
     TensorData td = resolve(n);
+    if (eb.split && n->kind != NodeKind::Tensor) materialized_[n.get()] = td;  // the other piece's pass reuses it
+    if (eb.split && !eb.inside_piece) {
+      std::vector<std::pair<size_t, size_t>> r;
+      for (size_t d = 0; d < td.layout.rank(); d++)
+        r.push_back(d == eb.split->axis ? std::make_pair(eb.split->start, eb.split->end) : std::make_pair(size_t(0), td.layout.shape[d]));
+      td.layout = td.layout.slice(r);
+    }
     v = eb.load(td);
   }
   eb.memo[n.get()] = v;
   return v;
 }
+
+namespace {
+// cat([A, B], axis) as Tensor::cat builds it (src/composite/cat.rs:3-41): slice_assign(resize(A, total), [len(A), total) on axis, B).
+bool match_cat2(const Node* n, NodeP* a, NodeP* b, size_t* axis) {
+  if (n->kind != NodeKind::SliceAssign || n->a->kind != NodeKind::Resize) return false;
+  const Node* rz = n->a.get();
+  const std::vector<size_t>& total = n->shape;
+  const std::vector<size_t>& sa = rz->a->shape;
+  const std::vector<size_t>& sb = n->b->shape;
+  if (rz->new_shape != total || rz->fill_shape != sa || sa.size() != total.size() || sb.size() != total.size()) return false;
+  int ax = -1;
+  for (size_t d = 0; d < total.size(); d++) {
+    if (sa[d] == total[d] && sb[d] == total[d] && n->ranges[d] == std::make_pair(size_t(0), total[d])) continue;
+    if (ax >= 0) return false;
+    if (sa[d] + sb[d] != total[d] || n->ranges[d] != std::make_pair(sa[d], total[d])) return false;
+    ax = int(d);
+  }
+  if (ax < 0) return false;
+  *a = rz->a;
+  *b = n->b;
+  *axis = size_t(ax);
+  return true;
+}
+
+const Node* find_cat2(const Node* n, int depth = 0) {
+  if (depth > 64) return nullptr;
+  NodeP a, b;
+  size_t axis;
+  if (match_cat2(n, &a, &b, &axis)) return n;
+  if (n->kind == NodeKind::ElementWise) return find_cat2(n->a.get(), depth + 1);
+  if (n->kind == NodeKind::PairWise) {
+    if (const Node* f = find_cat2(n->a.get(), depth + 1)) return f;
+    return find_cat2(n->b.get(), depth + 1);
+  }
+  return nullptr;
+}
+}  // namespace
 
 TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero) {
   TensorData td;
@@ -151,9 +200,12 @@ static std::string entry_name(const std::string& sig) {
   return buf;
 }
 
-wkf_kernel* Resolver::kernel(const std::string& sig, const std::string& body) {
+wkf_kernel* Resolver::kernel(const std::string& sig, const std::function<std::string()>& make_body) {
+  wkf_kernel* cached = nullptr;
+  check(wkf_module_find(dev_, sig.c_str(), &cached));
+  if (cached) return cached;  // the hot path: no source text is built
   const std::string entry = entry_name(sig);
-  const std::string src = "#define WKF_ENTRY " + entry + "\n" + body;
+  const std::string src = "#define WKF_ENTRY " + entry + "\n" + make_body();
   {
     std::lock_guard<std::mutex> lock(g_source_mu);
     g_sources.emplace(sig, src);
@@ -241,7 +293,275 @@ TensorData Resolver::resolve_root(const NodeP& root) {
   return out;
 }
 
+// ---- row kernels -----------------------------------------------------------------------------
+
+namespace {
+constexpr int kScalarBase = 1000;  // placeholder operand index of "scalar of stage s" until the operand count is known
+
+// A broadcast along the last axis of [an element-wise chain over] a reduce over the last axis of a
+// tensor of the same rows: returns that reduce node (and the chain, outermost first), else null.
+const Node* row_scalar_source(const Node* n, const std::vector<size_t>& shape, std::vector<const Node*>* chain) {
+  if (n->kind != NodeKind::MapLayout || n->map_kind != MapKind::Broadcast) return nullptr;
+  if (shape.empty() || n->axis0 != shape.size() - 1 || n->shape != shape) return nullptr;
+  const Node* cur = n->a.get();
+  while (cur->kind == NodeKind::ElementWise) {
+    if (chain) chain->push_back(cur);
+    cur = cur->a.get();
+  }
+  if (cur->kind != NodeKind::Reduce || cur->axis != shape.size() - 1 || cur->a->shape != shape) return nullptr;
+  return cur;
+}
+
+bool has_row_pattern(const Node* n, const std::vector<size_t>& shape, int depth = 0) {
+  if (depth > 64) return false;
+  if (row_scalar_source(n, shape, nullptr)) return true;
+  if (n->kind == NodeKind::ElementWise) return has_row_pattern(n->a.get(), shape, depth + 1);
+  if (n->kind == NodeKind::PairWise) return has_row_pattern(n->a.get(), shape, depth + 1) || has_row_pattern(n->b.get(), shape, depth + 1);
+  return false;
+}
+}  // namespace
+
+struct Resolver::RowBuild {
+  std::vector<size_t> shape;
+  std::vector<TensorData> operands;
+  std::vector<RowStage> stages;
+  std::map<const Node*, int> stage_of;  // reduce node -> stage
+  bool ok = true;
+};
+
+int Resolver::row_build(RowBuild& rb, Program& prog, std::map<const Node*, int>& memo, std::map<int, int>& loads, const NodeP& n) {
+  auto it = memo.find(n.get());
+  if (it != memo.end()) return it->second;
+  auto load = [&](int operand, DType dt) {
+    auto l = loads.find(operand);
+    if (l != loads.end()) return l->second;
+    Instr in;
+    in.op = Op::Load;
+    in.dtype = dt;
+    in.operand = operand;
+    prog.ins.push_back(in);
+    return loads[operand] = int(prog.ins.size()) - 1;
+  };
+  int v = -1;
+  std::vector<const Node*> chain;
+  if (const Node* red = row_scalar_source(n.get(), rb.shape, &chain)) {
+    int stage;
+    auto st = rb.stage_of.find(red);
+    if (st != rb.stage_of.end()) stage = st->second;
+    else {
+      // the stage's own expression first (it may create earlier stages), then the stage
+      RowStage rs;
+      rs.rop = red->rop;
+      std::map<const Node*, int> pmemo;
+      std::map<int, int> ploads;
+      rs.pre.result = row_build(rb, rs.pre, pmemo, ploads, red->a);
+      if (!rb.ok) return 0;
+      Instr ld;
+      ld.op = Op::Load;
+      ld.dtype = rs.pre.result_dtype();
+      ld.operand = 0;
+      rs.post.ins.push_back(ld);
+      rs.post.result = 0;
+      rb.stages.push_back(rs);
+      stage = int(rb.stages.size()) - 1;
+      rb.stage_of[red] = stage;
+    }
+    // the chain between the reduce and the broadcast is applied per element here (one scalar op per
+    // lane and row element costs nothing next to the loads and keeps one code path)
+    v = load(kScalarBase + stage, rb.stages[stage].post.result_dtype());
+    for (size_t i = chain.size(); i-- > 0;) {
+      const Node* c = chain[i];
+      if (c->op == Op::Sin || c->op == Op::Cos) rb.ok = false;
+      Instr in;
+      in.op = c->op;
+      in.a = v;
+      in.dtype = c->dtype;
+      if (is_const_op(c->op)) {
+        in.cslot = int(prog.consts.size());
+        prog.consts.push_back(c->constant);
+      }
+      prog.ins.push_back(in);
+      v = int(prog.ins.size()) - 1;
+    }
+  } else if (n->kind == NodeKind::ElementWise) {
+    if (n->op == Op::Sin || n->op == Op::Cos) rb.ok = false;  // would need the far-argument redo path
+    int a = row_build(rb, prog, memo, loads, n->a);
+    Instr in;
+    in.op = n->op;
+    in.a = a;
+    in.dtype = n->dtype;
+    if (is_const_op(n->op)) {
+      in.cslot = int(prog.consts.size());
+      prog.consts.push_back(n->constant);
+    }
+    prog.ins.push_back(in);
+    v = int(prog.ins.size()) - 1;
+  } else if (n->kind == NodeKind::PairWise && prog.ins.size() < 48) {
+    int a = row_build(rb, prog, memo, loads, n->a);
+    int b = row_build(rb, prog, memo, loads, n->b);
+    Instr in;
+    in.op = n->op;
+    in.a = a;
+    in.b = b;
+    in.dtype = n->dtype;
+    prog.ins.push_back(in);
+    v = int(prog.ins.size()) - 1;
+  } else {
+    TensorData td = resolve(n);
+    if (td.layout.shape != rb.shape) {
+      rb.ok = false;
+      return 0;
+    }
+    int k = -1;
+    for (size_t i = 0; i < rb.operands.size(); i++)
+      if (rb.operands[i].buffer.get() == td.buffer.get() && rb.operands[i].dtype == td.dtype && rb.operands[i].layout == td.layout) k = int(i);
+    if (k < 0) {
+      rb.operands.push_back(td);
+      k = int(rb.operands.size()) - 1;
+    }
+    v = load(k, td.dtype);
+  }
+  memo[n.get()] = v;
+  return v;
+}
+
+bool Resolver::try_row_kernel(const NodeP& root, TensorData* result) {
+  if (st_.fusion != FusionMode::Tree || root->shape.empty()) return false;
+  if (!has_row_pattern(root.get(), root->shape)) return false;
+  RowBuild rb;
+  rb.shape = root->shape;
+  Program final;
+  std::map<const Node*, int> memo;
+  std::map<int, int> loads;
+  final.result = row_build(rb, final, memo, loads, root);
+  if (!rb.ok || rb.stages.empty() || rb.operands.empty() || rb.operands.size() > 4 || rb.stages.size() > 4) return false;
+  const size_t R = rb.shape.size(), axis = R - 1, n = rb.shape[axis];
+  const size_t K = rb.operands.size();
+
+  RowSpec spec;
+  size_t max_elem = dtype_size(final.result_dtype());
+  for (const TensorData& td : rb.operands) max_elem = std::max(max_elem, dtype_size(td.dtype));
+  const int V = int(16 / max_elem);
+  if (n == 0 || n % V) return false;
+  std::vector<size_t> out_shape(rb.shape.begin(), rb.shape.end() - 1);
+  TensorData out = alloc(rb.shape, final.result_dtype(), false);
+  std::vector<std::vector<size_t>> ostr;
+  for (const TensorData& td : rb.operands) ostr.push_back(std::vector<size_t>(td.layout.strides.begin(), td.layout.strides.end() - 1));
+  ostr.push_back(std::vector<size_t>(out.layout.strides.begin(), out.layout.strides.end() - 1));
+  Space sp = coalesce(out_shape, ostr);
+  const size_t Ro = sp.shape.size();
+  if (Ro > 3) return false;
+  for (size_t k = 0; k < K; k++) {
+    const TensorData& td = rb.operands[k];
+    const size_t as = td.layout.strides[axis];
+    if (as > 1) return false;
+    if (as == 1) {
+      if (td.layout.offset % V) return false;
+      for (size_t d = 0; d < Ro; d++)
+        if (sp.strides[k][d] % V) return false;
+    }
+    if (td.layout.extent() > 0xffffffffull) return false;
+    spec.in.push_back({td.dtype, int(as)});
+  }
+  const size_t nvec = n / V;
+  int T = std::min(1024, pow2_ceil((nvec + 7) / 8));
+  if (nvec % T) return false;
+  const size_t NV = nvec / T;
+  if (NV > 16 || NV * V * K > 128) return false;
+  size_t nrows = 1;
+  for (size_t d : out_shape) nrows *= d;
+  if (nrows == 0) {
+    *result = out;
+    return true;
+  }
+  if (nrows > 0xffffffffull) return false;
+
+  // operand numbering: full operands 0..K-1, then the scalars
+  auto renumber = [&](Program& p) {
+    for (Instr& in : p.ins)
+      if (in.op == Op::Load && in.operand >= kScalarBase) in.operand = int(K) + (in.operand - kScalarBase);
+  };
+  for (RowStage& st : rb.stages) renumber(st.pre);
+  renumber(final);
+  spec.outer_rank = int(Ro);
+  spec.vec = V;
+  spec.threads_per_row = T;
+  spec.block = std::max(256, T);
+  spec.vectors_per_lane = int(NV);
+  spec.stages = rb.stages;
+  spec.final = final;
+  spec.out_dtype = final.result_dtype();
+  spec.exact_math = st_.exact_math;
+
+  RowArgs args;
+  args.nrows = uint32_t(nrows);
+  for (size_t d = 0; d < Ro; d++) args.oshape.push_back(to_u32(sp.shape[d], "shape"));
+  for (size_t k = 0; k <= K; k++) {
+    const TensorData& td = k < K ? rb.operands[k] : out;
+    args.ptrs.push_back(element_ptr(td));
+    args.offsets.push_back(to_u32(td.layout.offset, "offset"));
+    std::vector<uint32_t> st;
+    for (size_t d = 0; d < Ro; d++) st.push_back(to_u32(sp.strides[k][d], "stride"));
+    args.ostrides.push_back(st);
+  }
+  for (const RowStage& st : rb.stages) {
+    args.consts.insert(args.consts.end(), st.pre.consts.begin(), st.pre.consts.end());
+    args.consts.insert(args.consts.end(), st.post.consts.begin(), st.post.consts.end());
+  }
+  args.consts.insert(args.consts.end(), final.consts.begin(), final.consts.end());
+
+  std::string sig = row_signature(spec);
+  wkf_kernel* k = kernel(sig, [&] { return row_source(spec); });
+  LaunchRecord r;
+  r.kind = "row";
+  r.signature = sig;
+  const size_t rpb = size_t(spec.block / T);
+  r.grid[0] = to_u32((nrows + rpb - 1) / rpb, "grid");
+  r.block[0] = uint32_t(spec.block);
+  std::ostringstream d;
+  d << "rows=" << nrows << " n=" << n << " vec=" << V << " threads_per_row=" << T << " vectors_per_lane=" << NV << " stages="
+    << rb.stages.size() << " operands=" << K + 1;
+  r.detail = d.str();
+  record(std::move(r), k, row_pack_args(spec, args));
+  *result = out;
+  return true;
+}
+
 TensorData Resolver::run_map(const NodeP& root) {
+  {
+    TensorData fused;
+    if (try_row_kernel(root, &fused)) return fused;
+  }
+  // A consumer of cat([A, B]) runs once per piece and writes straight into its part of the result,
+  // instead of copying the pieces together first and reading the copy back (rope's rotate_half).
+  if (st_.fusion == FusionMode::Tree && root->kind != NodeKind::SliceAssign) {
+    if (const Node* cat = find_cat2(root.get())) {
+      NodeP pa, pb;
+      size_t axis = 0;
+      match_cat2(cat, &pa, &pb, &axis);
+      const size_t mid = pa->shape[axis], total = cat->shape[axis];
+      TensorData out;
+      for (int part = 0; part < 2; part++) {
+        CatPiece piece;
+        piece.cat = cat;
+        piece.piece = part == 0 ? pa : pb;
+        piece.axis = axis;
+        piece.start = part == 0 ? 0 : mid;
+        piece.end = part == 0 ? mid : total;
+        ExprBuilder eb;
+        eb.split = &piece;
+        eb.prog.result = build(eb, root, pairwise_budget_for_map());
+        if (part == 0) out = alloc(root->shape, eb.prog.result_dtype(), false);
+        std::vector<std::pair<size_t, size_t>> r;
+        for (size_t d = 0; d < root->shape.size(); d++)
+          r.push_back(d == axis ? std::make_pair(piece.start, piece.end) : std::make_pair(size_t(0), root->shape[d]));
+        TensorData view = out;
+        view.layout = out.layout.slice(r);
+        if (piece.end > piece.start) launch_map(eb.prog, eb.operands, view, false);
+      }
+      return out;
+    }
+  }
   ExprBuilder eb;
   int v = build(eb, root, pairwise_budget_for_map());
   eb.prog.result = v;
@@ -343,7 +663,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   args.consts = prog.consts;
 
   std::string sig = map_signature(spec);
-  wkf_kernel* k = kernel(sig, map_source(spec));
+  wkf_kernel* k = kernel(sig, [&] { return map_source(spec); });
   LaunchRecord r;
   r.kind = "map";
   r.signature = sig;
@@ -510,7 +830,7 @@ TensorData Resolver::run_reduce(const NodeP& rn, const std::vector<const Node*>&
   args.consts.insert(args.consts.end(), post.consts.begin(), post.consts.end());
 
   std::string sig = reduce_signature(spec);
-  wkf_kernel* k = kernel(sig, reduce_source(spec));
+  wkf_kernel* k = kernel(sig, [&] { return reduce_source(spec); });
   r.signature = sig;
   r.detail = d.str();
   record(std::move(r), k, reduce_pack_args(spec, args));

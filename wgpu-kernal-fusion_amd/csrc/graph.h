@@ -4,6 +4,7 @@
 // and the run_with_query methods of the reference's kernel objects.
 #pragma once
 
+#include <functional>
 #include <map>
 #include <set>
 #include <string>
@@ -42,7 +43,16 @@ class Resolver {
  private:
   TensorData resolve(const NodeP& n);
   TensorData resolve_uncached(const NodeP& n);
+  // When a map kernel consumes cat([A, B], axis), the kernel is run once per piece: the cat
+  // node stands for A (or B) and every other operand is sliced to that piece's range.
+  struct CatPiece {
+    const Node* cat = nullptr;   // the slice_assign node that completes the cat
+    NodeP piece;                 // A or B
+    size_t axis = 0, start = 0, end = 0;
+  };
   struct ExprBuilder {
+    const CatPiece* split = nullptr;
+    bool inside_piece = false;
     Program prog;
     std::vector<TensorData> operands;
     std::map<const Node*, int> memo;
@@ -56,6 +66,12 @@ class Resolver {
   int pairwise_budget_for_reduce() const { return st_.fusion == FusionMode::Tree ? 1 << 20 : 0; }
 
   TensorData run_map(const NodeP& root);
+  // Row kernels (codegen.h, RowSpec): tried first for a map whose operands include last-axis
+  // reductions of the same rows broadcast back along that axis.  Returns false when the pattern
+  // or the layouts do not fit; the caller then takes the ordinary path.
+  struct RowBuild;
+  bool try_row_kernel(const NodeP& root, TensorData* out);
+  int row_build(RowBuild& rb, Program& prog, std::map<const Node*, int>& memo, std::map<int, int>& loads, const NodeP& n);
   TensorData run_reduce(const NodeP& reduce, const std::vector<const Node*>& post_chain);
   TensorData run_matmul(const NodeP& n);
   TensorData run_map_layout(const NodeP& n);
@@ -67,7 +83,7 @@ class Resolver {
   TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero);
   TensorData make_contiguous(const TensorData& td);
   void record(LaunchRecord&& r, wkf_kernel* k, const std::vector<unsigned char>& args);
-  wkf_kernel* kernel(const std::string& sig, const std::string& src);
+  wkf_kernel* kernel(const std::string& sig, const std::function<std::string()>& make_body);
 
   wkf_device* dev_;
   Settings st_;

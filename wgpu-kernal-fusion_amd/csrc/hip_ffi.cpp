@@ -445,6 +445,15 @@ int wkf_module_get(wkf_device* dev, const char* signature, const char* hip_sourc
   return WKF_OK;
 }
 
+int wkf_module_find(wkf_device* dev, const char* signature, wkf_kernel** out) {
+  if (!dev || !signature || !out) return fail(WKF_ERR_INVALID_ARG, "wkf_module_find: null argument");
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  auto it = dev->kernels.find(signature);
+  *out = it == dev->kernels.end() ? nullptr : it->second;
+  if (*out) dev->n_mem++;
+  return WKF_OK;
+}
+
 int wkf_module_stats(wkf_device* dev, uint64_t* compiled, uint64_t* disk_hits, uint64_t* mem_hits) {
   if (!dev) return fail(WKF_ERR_INVALID_ARG, "wkf_module_stats: null device");
   if (compiled) *compiled = dev->n_compiled;
