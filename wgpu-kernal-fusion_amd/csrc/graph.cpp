@@ -631,7 +631,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   spec.prog = prog;
   spec.math = st_.exact_math ? MathPolicy::Exact : MathPolicy::Stored;
   const size_t nwork = numel / vec;
-  spec.unroll = nwork >= (1u << 20) ? 4 : nwork >= (1u << 16) ? 2 : 1;
+  spec.unroll = nwork >= (1u << 20) ? st_.map_unroll : nwork >= (1u << 16) ? 2 : 1;
   size_t bytes = 0;
   std::vector<size_t> cstrides = Layout::contiguous_strides(sp.shape);
   for (size_t k = 0; k < N; k++) {

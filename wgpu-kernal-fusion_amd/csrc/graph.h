@@ -30,6 +30,7 @@ struct LaunchRecord {
 struct Settings {
   FusionMode fusion = FusionMode::Tree;
   bool timing = true;             // record a hipEvent pair around every launch
+  int map_unroll = 4;             // work items per thread in large map kernels (WKF_MAP_UNROLL overrides: 1, 2, 4, 8)
   bool exact_math = false;        // every transcendental through an f64 core (MathPolicy::Exact)
   size_t nontemporal_bytes = size_t(32) << 20;  // map kernels moving at least this much use streaming loads/stores
 };

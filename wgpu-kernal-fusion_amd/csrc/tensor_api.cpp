@@ -88,7 +88,18 @@ std::unordered_map<wkf_device*, Settings> g_settings;
 
 Settings settings_for(wkf_device* dev) {
   std::lock_guard<std::mutex> lock(g_settings_mu);
-  return g_settings[dev];
+  auto it = g_settings.find(dev);
+  if (it == g_settings.end()) {
+    // tuning knobs read once per device
+    Settings st;
+    if (const char* u = getenv("WKF_MAP_UNROLL")) {
+      int v = atoi(u);
+      if (v == 1 || v == 2 || v == 4 || v == 8) st.map_unroll = v;
+    }
+    if (const char* nt = getenv("WKF_NONTEMPORAL_BYTES")) st.nontemporal_bytes = size_t(atoll(nt));
+    it = g_settings.emplace(dev, st).first;
+  }
+  return it->second;
 }
 
 // Runs `f`, mapping exceptions to status codes + wkf_last_error().
@@ -389,6 +400,7 @@ int wkf_device_set_fusion(wkf_device* dev, int mode) {
   return guarded([&] {
     need(dev, "wkf_device_set_fusion");
     if (mode != WKF_FUSION_REFERENCE && mode != WKF_FUSION_TREE) invalid("unknown fusion mode");
+    settings_for(dev);  // creates the entry (and reads the tuning knobs) on first use
     std::lock_guard<std::mutex> lock(g_settings_mu);
     g_settings[dev].fusion = FusionMode(mode);
   });
@@ -399,6 +411,7 @@ int wkf_device_get_fusion(wkf_device* dev) { return int(settings_for(dev).fusion
 int wkf_device_set_timing(wkf_device* dev, int enabled) {
   return guarded([&] {
     need(dev, "wkf_device_set_timing");
+    settings_for(dev);  // creates the entry (and reads the tuning knobs) on first use
     std::lock_guard<std::mutex> lock(g_settings_mu);
     g_settings[dev].timing = enabled != 0;
   });
@@ -407,6 +420,7 @@ int wkf_device_set_timing(wkf_device* dev, int enabled) {
 int wkf_device_set_exact_math(wkf_device* dev, int exact) {
   return guarded([&] {
     need(dev, "wkf_device_set_exact_math");
+    settings_for(dev);
     std::lock_guard<std::mutex> lock(g_settings_mu);
     g_settings[dev].exact_math = exact != 0;
   });
