@@ -156,6 +156,35 @@ def test_strided_and_broadcast_operands(gpu):
         assert_ulp(g, w.to_numpy(), 0, f"view {i}")
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+def test_transposed_operands_take_the_tiled_kernel(gpu, dtype):
+    # inputs that are unit-stride along another dimension than the output go through a 64 x 64 LDS tile
+    api = HipAPI(gpu)
+    a = data((300, 523), -2, 2, dtype, 21)
+    b = data((523, 300), -2, 2, dtype, 22)
+    c = data((5, 130, 200), -2, 2, dtype, 23)
+    d = data((200, 5, 130), -2, 2, dtype, 24)
+
+    def progs(ta, tb, tc, td):
+        return [ta.transpose(0, 1) + 1.0,                              # ragged edge tiles on both sides
+                ta.transpose(0, 1) * tb,                               # one crossed, one straight operand
+                (ta.transpose(0, 1) + tb) - ta.transpose(0, 1) * 0.5,  # the crossed operand is read once
+                tc.transpose(1, 2) * 2.0,                              # batch dim in front
+                tc.transpose(0, 2).transpose(1, 2) + td,               # [200, 5, 130] from [5, 130, 200]
+                ta.slice([(3, 290), (10, 500)]).transpose(0, 1) * tb.slice([(10, 500), (3, 290)])]
+
+    got = hip_values_many(progs(api.tensor(a), api.tensor(b), api.tensor(c), api.tensor(d)))
+    want = progs(OTensor(a), OTensor(b), OTensor(c), OTensor(d))
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert np.array_equal(g, w.to_numpy()), f"program {i}"
+    if dtype == np.float32:
+        far = a.copy()
+        far[::7, ::5] *= 1e6  # some arguments beyond the fast trig range
+        g = hip_values(api.tensor(far).transpose(0, 1).sin() + api.tensor(b))
+        w = (OTensor(far).transpose(0, 1).sin() + OTensor(b)).to_numpy()
+        assert_ulp(g, w, 2)
+
+
 def test_same_results_under_both_fusion_modes(gpu):
     a, b = data((64, 96), -2, 2, np.float32, 11), data((64, 96), 0.5, 2, np.float32, 12)
     api = HipAPI(gpu)
@@ -183,7 +212,10 @@ def test_same_results_under_both_fusion_modes(gpu):
 
 RED_SHAPES = [((1,), 0), ((5,), 0), ((4096,), 0), ((3, 2), 0), ((3, 2), 1), ((1, 7), 1), ((7, 1), 1), ((64, 64), 0),
               ((64, 64), 1), ((9, 1000), 1), ((1000, 9), 0), ((3, 100003), 1), ((5, 6, 7), 0), ((5, 6, 7), 1),
-              ((5, 6, 7), 2), ((2, 3, 4, 5), 2), ((300, 8192), 1), ((33, 2048), 1), ((16, 4096), 1), ((2, 65536), 1)]
+              ((5, 6, 7), 2), ((2, 3, 4, 5), 2), ((300, 8192), 1), ((33, 2048), 1), ((16, 4096), 1), ((2, 65536), 1),
+              # few outputs over a long axis: folded in two launches; lanes own 4 (f32) / 8 (f16) columns
+              ((4096, 160), 0), ((8192, 512), 0), ((4, 262144), 1), ((4100, 36), 0), ((3, 4096, 20), 1), ((4096, 6, 8), 0),
+              ((4098, 66), 0)]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
@@ -231,6 +263,27 @@ def test_reductions_of_views_and_rank0(gpu):
         assert g.shape == w.to_numpy().shape
         assert np.allclose(g, w.to_numpy(), rtol=1e-5, atol=1e-6), f"view reduce {i}"
     assert got[5].shape == () and got[6].shape == ()
+
+
+def test_long_axis_reductions_of_views(gpu):
+    api = HipAPI(gpu)
+    a = data((4096, 96), -1, 1, np.float32, 16)
+    b = data((4, 6, 4096, 9), -1, 1, np.float32, 17)
+
+    def progs(ta, tb):
+        return [ta.transpose(0, 1).sum(1),                              # strided axis, unit-stride outputs: sliced in two launches
+                (ta.transpose(0, 1) * 0.5).max(1) + 1.0,
+                ta.slice([(0, 4096), (8, 72)]).sum(0),
+                tb.slice([(0, 3), (0, 5), (0, 4096), (0, 7)]).sum(2),   # three outer dims that do not merge: one launch
+                tb.sum(2), tb.transpose(2, 3).min(3)]
+
+    got = hip_values_many(progs(api.tensor(a), api.tensor(b)))
+    want = progs(OTensor(a), OTensor(b))
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert g.shape == w.to_numpy().shape
+        # 1e-5 relative to the sum of magnitudes (about 2000 here)
+        assert np.allclose(g, w.to_numpy(), rtol=1e-5, atol=1e-3), f"view reduce {i}"
+    assert np.array_equal(got[5], want[5].to_numpy())
 
 
 def test_reduce_seeds_and_empty_axes(gpu):

@@ -220,6 +220,28 @@ def test_tree_mode_fuses_pair_wise_trees_and_copies(wkf, planner):
     assert all(k == "map" for k in kinds) and len(kinds) <= 8
 
 
+def test_few_outputs_over_a_long_axis_fold_in_two_launches(wkf, planner):
+    # the reference always puts one workgroup on one output (src/reduce.rs:316-346); here a long axis with too
+    # few outputs to fill the chip is cut into slices whose f32 partial folds a second launch finishes
+    x = wkf.Tensor.new(planner, np.zeros((8192, 512), dtype=np.float32))
+    t = (x * 2.0).sum(0) + 1.0
+    assert _kinds(t) == ["red_col", "red_col"]
+    first, second = t.kernels()
+    assert first.detail.endswith("partial") and "vec=4" in first.detail and "|raw" in first.signature
+    assert "multiply_const" in first.signature and "add_const" not in first.signature
+    assert "pre:load:f32@0->0|" in second.signature and "add_const" in second.signature and "fold:f32" in second.signature
+    h = wkf.Tensor.new(planner, np.zeros((4, 262144), dtype=np.float16)).max(1)
+    assert _kinds(h) == ["red_row", "red_row"]
+    assert "fold:f16" in h.kernels()[1].signature and "in:f32" in h.kernels()[1].signature
+    # an axis length without a power-of-two factor is not cut
+    assert _kinds(wkf.Tensor.new(planner, np.zeros((3, 100003), dtype=np.float32)).sum(1)) == ["red_row"]
+    planner.set_fusion(wkf.FUSION_REFERENCE)
+    try:
+        assert _kinds(wkf.Tensor.new(planner, np.zeros((8192, 512), dtype=np.float32)).sum(0)) == ["red_col"]
+    finally:
+        planner.set_fusion(wkf.FUSION_TREE)
+
+
 def test_one_binary_serves_every_size_and_constant(wkf, planner):
     before = planner.module_stats()
     t1 = (_x(wkf, planner, (256, 256)) * 3.0) + 5.0

@@ -174,10 +174,99 @@ std::string map_signature(const MapSpec& s) {
   for (const auto& i : s.in) o << dtype_name(i.dtype) << (i.linear ? 'L' : 'S') << i.inner_stride << ',';
   o << "|out:" << dtype_name(s.out.dtype) << (s.out.linear ? 'L' : 'S') << s.out.inner_stride;
   o << "|m" << int(s.math) << "|" << s.prog.signature();
+  if (s.tile_dim >= 0) {
+    o << "|tile" << s.tile_dim << ':';
+    for (size_t k = 0; k < s.in.size(); k++) o << (s.crossed[k] ? 'x' : '-');
+  }
   return o.str();
 }
 
+namespace {
+// out = expr(inputs) where some inputs run along `tile_dim` and the output along the last dimension.
+std::string map_tiled_source(const MapSpec& s) {
+  const int N = int(s.in.size()) + 1;
+  const int R = s.rank, TA = s.tile_dim, TB = s.rank - 1;
+  const int NC = s.prog.consts.empty() ? 1 : int(s.prog.consts.size());
+  const int PER = kMapTile * kMapTile / kMapBlock;  // tile rows per thread
+  std::ostringstream o;
+  o << kPrelude;
+  if (uses_math(s.prog, s.math)) o << kMath;
+  o << "struct Args { void* p[" << N << "]; u32 nwork; u32 shape[" << R << "]; u32 off[" << N << "]; u32 stride[" << N
+    << "][" << R << "]; float c[" << NC << "]; };\n";
+  std::vector<DType> types;
+  for (const auto& i : s.in) types.push_back(i.dtype);
+  emit_program(o, s.prog, "wkf_expr", types, s.math);
+  const bool trig = uses_trig(s.prog, s.math);
+  auto dt = [&](int k) { return k < N - 1 ? s.in[k].dtype : s.out.dtype; };
+  auto ptr = [&](int k) {
+    return std::string("((") + (k < N - 1 ? "const " : "") + ctype(dt(k)) + "*)a.p[" + std::to_string(k) + "])";
+  };
+  o << "extern \"C\" __global__ void __launch_bounds__(" << kMapBlock << ") WKF_ENTRY(const Args a) {\n";
+  for (int k = 0; k < N - 1; k++)
+    if (s.crossed[k])  // the padding keeps both the row-wise writes and the column-wise reads free of bank conflicts
+      o << "  __shared__ " << ctype(dt(k)) << " tile" << k << "[" << kMapTile << "][" << kMapTile + (dtype_size(dt(k)) == 2 ? 2 : 1) << "];\n";
+  o << "  const u32 tx = threadIdx.x & 63u, ty = threadIdx.x >> 6;\n";
+  o << "  const u32 A = a.shape[" << TA << "], B = a.shape[" << TB << "];\n";
+  o << "  const u32 tiles_a = (A + 63u) / 64u, tiles_b = (B + 63u) / 64u;\n";
+  o << "  u32 rem = blockIdx.x;\n";
+  o << "  const u32 b0 = (rem % tiles_b) * 64u; rem /= tiles_b;\n";
+  o << "  const u32 a0 = (rem % tiles_a) * 64u; rem /= tiles_a;\n";
+  std::vector<int> others;
+  for (int d = R - 2; d >= 0; d--)
+    if (d != TA) others.push_back(d);
+  for (size_t i = 0; i < others.size(); i++) {
+    const int d = others[i];
+    if (i + 1 < others.size()) o << "  const u32 i" << d << " = rem % a.shape[" << d << "]; rem /= a.shape[" << d << "];\n";
+    else o << "  const u32 i" << d << " = rem;\n";
+  }
+  for (int k = 0; k < N; k++) {
+    o << "  const u32 base" << k << " = a.off[" << k << "]";
+    for (int d : others) o << " + i" << d << " * a.stride[" << k << "][" << d << "]";
+    o << ";\n";
+  }
+  // phase 1: crossed inputs, lanes along tile_dim (indices clamped so that every load is unconditional)
+  for (int k = 0; k < N - 1; k++) {
+    if (!s.crossed[k]) continue;
+    o << "  {\n    " << ctype(dt(k)) << " r[" << PER << "];\n";
+    o << "    const u32 aa = min(a0 + tx, A - 1u);\n";
+    o << "#pragma unroll\n    for (int j = 0; j < " << PER << "; j++) {\n";
+    o << "      const u32 bb = min(b0 + ty * " << PER << "u + j, B - 1u);\n";
+    o << "      r[j] = " << ptr(k) << "[base" << k << " + aa * a.stride[" << k << "][" << TA << "] + bb * a.stride[" << k << "]["
+      << TB << "]];\n    }\n";
+    o << "#pragma unroll\n    for (int j = 0; j < " << PER << "; j++) tile" << k << "[ty * " << PER << "u + j][tx] = r[j];\n  }\n";
+  }
+  o << "  __syncthreads();\n";
+  // phase 2: lanes along the last dim
+  o << "  const u32 bb = min(b0 + tx, B - 1u);\n";
+  o << "  const bool b_live = b0 + tx < B;\n";
+  for (int k = 0; k < N - 1; k++) {
+    if (s.crossed[k]) continue;
+    o << "  " << ctype(dt(k)) << " s" << k << "[" << PER << "];\n";
+    o << "#pragma unroll\n  for (int j = 0; j < " << PER << "; j++) {\n";
+    o << "    const u32 aa = min(a0 + ty * " << PER << "u + j, A - 1u);\n";
+    o << "    s" << k << "[j] = " << ptr(k) << "[base" << k << " + aa * a.stride[" << k << "][" << TA << "] + bb * a.stride[" << k
+      << "][" << TB << "]];\n  }\n";
+  }
+  o << "#pragma unroll\n  for (int j = 0; j < " << PER << "; j++) {\n";
+  o << "    const u32 aa = a0 + ty * " << PER << "u + j;\n";
+  std::ostringstream call;
+  for (int k = 0; k < N - 1; k++) {
+    if (s.crossed[k]) call << "tile" << k << "[tx][ty * " << PER << "u + j], ";
+    else call << "s" << k << "[j], ";
+  }
+  call << "a.c";
+  if (trig) o << "    bool far = false;\n";
+  o << "    " << ctype(s.out.dtype) << " v = wkf_expr(" << call.str() << (trig ? ", far" : "") << ");\n";
+  if (trig) o << "    if (__builtin_expect(far, 0)) v = wkf_expr_far(" << call.str() << ");\n";
+  o << "    if (b_live && aa < A) " << ptr(N - 1) << "[base" << N - 1 << " + aa * a.stride[" << N - 1 << "][" << TA
+    << "] + bb * a.stride[" << N - 1 << "][" << TB << "]] = v;\n";
+  o << "  }\n}\n";
+  return o.str();
+}
+}  // namespace
+
 std::string map_source(const MapSpec& s) {
+  if (s.tile_dim >= 0) return map_tiled_source(s);
   const int N = int(s.in.size()) + 1;  // operands incl. out
   const int R = s.rank, V = s.vec, U = s.unroll;
   const int NC = s.prog.consts.empty() ? 1 : int(s.prog.consts.size());
@@ -345,9 +434,10 @@ std::string reduce_signature(const ReduceSpec& s) {
   std::ostringstream o;
   o << (s.shape == ReduceShape::Row ? "red_row" : "red_col") << "|gfx950|" << reduce_name(s.rop) << "|or" << s.outer_rank
     << "|v" << s.vec << "|t" << s.threads_per_row << "|b" << s.block << "|u" << s.unroll << "|w" << s.waves << "|in:";
-  for (const auto& i : s.in) o << dtype_name(i.dtype) << 'a' << i.axis_stride << ',';
-  o << "|out:" << dtype_name(s.out_dtype) << "|m" << int(s.math_pre) << int(s.math_post) << "|pre:" << s.pre.signature()
-    << "|post:" << s.post.signature();
+  for (const auto& i : s.in) o << dtype_name(i.dtype) << 'a' << i.axis_stride << 'i' << i.inner_stride << ',';
+  o << "|out:" << dtype_name(s.out_dtype) << "|m" << int(s.math_pre) << int(s.math_post) << "|pre:" << s.pre.signature();
+  if (s.raw_out) o << "|raw";
+  else o << "|fold:" << dtype_name(s.fold_dtype) << "|post:" << s.post.signature();
   return o.str();
 }
 
@@ -357,9 +447,10 @@ std::string reduce_source(const ReduceSpec& s) {
   const int NCpre = int(s.pre.consts.size());
   const int NC = std::max(1, NCpre + int(s.post.consts.size()));
   const DType pre_dt = s.pre.result_dtype();
+  const bool raw = s.raw_out;
   std::ostringstream o;
   o << kPrelude;
-  if (uses_math(s.pre, s.math_pre) || uses_math(s.post, s.math_post)) o << kMath;
+  if (uses_math(s.pre, s.math_pre) || (!raw && uses_math(s.post, s.math_post))) o << kMath;
   o << fold_macro(s.rop);
   o << kReduceHelpers;
   o << "struct Args { void* p[" << N + 1 << "]; u32 nrows; u32 n; u32 nvec; u32 oshape[" << std::max(1, Ro)
@@ -368,7 +459,7 @@ std::string reduce_source(const ReduceSpec& s) {
   std::vector<DType> types;
   for (const auto& i : s.in) types.push_back(i.dtype);
   emit_program(o, s.pre, "wkf_pre", types, s.math_pre);
-  emit_program(o, s.post, "wkf_post", {pre_dt}, s.math_post);
+  if (!raw) emit_program(o, s.post, "wkf_post", {s.fold_dtype}, s.math_post);
 
   auto unravel = [&](const char* row, const char* ind) {
     // i_d = index along outer dim d of output element `row`
@@ -387,9 +478,12 @@ std::string reduce_source(const ReduceSpec& s) {
   auto ptr = [&](int k) { return std::string("((const ") + ctype(s.in[k].dtype) + "*)a.p[" + std::to_string(k) + "])"; };
   // the folded value is rounded to the tensor dtype, then `post` runs in that dtype
   // A post chain with sin / cos runs once per output, so it simply takes the far variant.
-  std::string store_value = std::string(uses_trig(s.post, s.math_post) ? "wkf_post_far((" : "wkf_post((") + ctype(pre_dt) + ")acc, a.c + " +
-                            std::to_string(NCpre) + ")";
-  std::string out_ptr = std::string("((") + ctype(s.out_dtype) + "*)a.p[" + std::to_string(N) + "])";
+  auto store_value = [&](const std::string& acc) {
+    if (raw) return acc;
+    return std::string(uses_trig(s.post, s.math_post) ? "wkf_post_far((" : "wkf_post((") + ctype(s.fold_dtype) + ")" + acc +
+           ", a.c + " + std::to_string(NCpre) + ")";
+  };
+  std::string out_ptr = std::string("((") + ctype(raw ? DType::F32 : s.out_dtype) + "*)a.p[" + std::to_string(N) + "])";
 
   if (s.shape == ReduceShape::Row) {
     const int T = s.threads_per_row, V = s.vec, U = s.unroll, B = s.block;
@@ -463,19 +557,20 @@ std::string reduce_source(const ReduceSpec& s) {
       o << "  acc = wkf_partial[first_wave];\n";
       o << "  for (u32 w = 1; w < " << WPR << "u; w++) acc = WKF_FOLD(wkf_partial[first_wave + w], acc);\n";
     }
-    o << "  if (live && t == 0u) " << out_ptr << "[" << base_expr(N) << "] = " << store_value << ";\n";
+    o << "  if (live && t == 0u) " << out_ptr << "[" << base_expr(N) << "] = " << store_value("acc") << ";\n";
     o << "}\n";
   } else {
-    const int W = s.waves;
+    // Each lane owns V neighbouring outputs of the LAST outer dim (one 16-byte load per axis step when
+    // V > 1); the W waves of the block walk the axis W steps apart, U steps in flight per wave.
+    const int W = s.waves, V = s.vec, U = s.unroll;
     o << "extern \"C\" __global__ void __launch_bounds__(" << 64 * W << ") WKF_ENTRY(const Args a) {\n";
-    if (W > 1) o << "  __shared__ float wkf_partial[" << W << "][64];\n";
+    if (W > 1) o << "  __shared__ float wkf_partial[" << W << "][" << V << "][64];\n";
     o << "  const u32 lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;\n";
-    // The 64 lanes of a wave sit on 64 neighbouring positions of the LAST outer dim.
     if (Ro == 0) {
       o << "  const bool live = lane == 0u && blockIdx.x == 0u;\n";
     } else {
-      o << "  const u32 ntile = (a.oshape[" << Ro - 1 << "] + 63u) / 64u;\n";
-      o << "  const u32 col = (blockIdx.x % ntile) * 64u + lane;\n";
+      o << "  const u32 ntile = (a.oshape[" << Ro - 1 << "] + " << 64 * V - 1 << "u) / " << 64 * V << "u;\n";
+      o << "  const u32 col = ((blockIdx.x % ntile) * 64u + lane) * " << V << "u;\n";
       o << "  const bool live = col < a.oshape[" << Ro - 1 << "];\n";
       o << "  const u32 i" << Ro - 1 << " = live ? col : 0u;\n";
       if (Ro > 1) {
@@ -487,25 +582,73 @@ std::string reduce_source(const ReduceSpec& s) {
     }
     for (int k = 0; k < N; k++)
       o << "  const " << ctype(s.in[k].dtype) << "* q" << k << " = " << ptr(k) << " + (" << base_expr(k) << ");\n";
-    o << "  float acc = WKF_SEED;\n";
-    o << "  for (u32 k = wave; k < a.n; k += " << W << "u) {\n";
-    {
-      const bool trig = uses_trig(s.pre, s.math_pre);
-      std::ostringstream call;
-      for (int k = 0; k < N; k++) call << "q" << k << "[k * a.astride[" << k << "]], ";
-      call << "a.c";
-      if (trig) o << "    bool far = false;\n";
-      o << "    " << ctype(pre_dt) << " t = wkf_pre(" << call.str() << (trig ? ", far" : "") << ");\n";
-      if (trig) o << "    if (__builtin_expect(far, 0)) t = wkf_pre_far(" << call.str() << ");\n";
-      o << "    acc = WKF_FOLD((float)t, acc);\n  }\n";
+    o << "  float acc[" << V << "];\n";
+    o << "  for (int e = 0; e < " << V << "; e++) acc[e] = WKF_SEED;\n";
+    const bool trig = uses_trig(s.pre, s.math_pre);
+    auto wide = [&](int k) { return V > 1 && s.in[k].inner_stride == 1; };
+    auto emit_step = [&](int j1, const std::string& ind) {
+      for (int j = 0; j < j1; j++)
+        for (int k = 0; k < N; k++) {
+          std::string vt = wide(k) ? vtype(s.in[k].dtype, V) : ctype(s.in[k].dtype);
+          std::string at = "q" + std::to_string(k) + " + (k + " + std::to_string(j * W) + "u) * a.astride[" + std::to_string(k) + "]";
+          o << ind << "const " << vt << " r" << k << "_" << j << " = ";
+          if (wide(k)) o << "__builtin_nontemporal_load((const " << vt << "*)(" << at << "));\n";
+          else o << "*(" << at << ");\n";
+        }
+      for (int j = 0; j < j1; j++)
+        for (int e = 0; e < V; e++) o << ind << ctype(pre_dt) << " t" << j << "_" << e << ";\n";
+      if (trig) o << ind << "bool far = false;\n";
+      auto values = [&](bool far_variant, const std::string& ind2) {
+        for (int j = 0; j < j1; j++)
+          for (int e = 0; e < V; e++) {
+            o << ind2 << "t" << j << "_" << e << " = wkf_pre" << (far_variant ? "_far" : "") << "(";
+            for (int k = 0; k < N; k++) {
+              o << "r" << k << "_" << j;
+              if (wide(k)) o << "[" << e << "]";
+              o << ", ";
+            }
+            o << "a.c" << (trig && !far_variant ? ", far" : "") << ");\n";
+          }
+      };
+      values(false, ind);
+      if (trig) {
+        o << ind << "if (__builtin_expect(far, 0)) {\n";
+        values(true, ind + "  ");
+        o << ind << "}\n";
+      }
+      for (int j = 0; j < j1; j++)
+        for (int e = 0; e < V; e++) o << ind << "acc[" << e << "] = WKF_FOLD((float)t" << j << "_" << e << ", acc[" << e << "]);\n";
+    };
+    o << "  u32 k = wave;\n";
+    if (U > 1) {
+      o << "  for (; k + " << (U - 1) * W << "u < a.n; k += " << U * W << "u) {\n";
+      emit_step(U, "    ");
+      o << "  }\n";
     }
+    o << "  for (; k < a.n; k += " << W << "u) {\n";
+    emit_step(1, "    ");
+    o << "  }\n";
+    auto emit_store = [&](const std::string& ind) {
+      if (V == 1) {
+        o << ind << "if (live) " << out_ptr << "[" << base_expr(N) << "] = " << store_value("acc[0]") << ";\n";
+        return;
+      }
+      const DType odt = raw ? DType::F32 : s.out_dtype;
+      o << ind << "if (live) {\n";
+      o << ind << "  " << vtype(odt, V) << " ov;\n";
+      for (int e = 0; e < V; e++) o << ind << "  ov[" << e << "] = " << store_value("acc[" + std::to_string(e) + "]") << ";\n";
+      o << ind << "  *(" << vtype(odt, V) << "*)(" << out_ptr << " + (" << base_expr(N) << ")) = ov;\n";
+      o << ind << "}\n";
+    };
     if (W > 1) {
-      o << "  wkf_partial[wave][lane] = acc;\n  __syncthreads();\n";
+      o << "  for (int e = 0; e < " << V << "; e++) wkf_partial[wave][e][lane] = acc[e];\n  __syncthreads();\n";
       o << "  if (wave == 0u) {\n";
-      o << "    for (u32 w = 1; w < " << W << "u; w++) acc = WKF_FOLD(wkf_partial[w][lane], acc);\n";
-      o << "    if (live) " << out_ptr << "[" << base_expr(N) << "] = " << store_value << ";\n  }\n";
+      o << "    for (u32 w = 1; w < " << W << "u; w++)\n";
+      o << "      for (int e = 0; e < " << V << "; e++) acc[e] = WKF_FOLD(wkf_partial[w][e][lane], acc[e]);\n";
+      emit_store("    ");
+      o << "  }\n";
     } else {
-      o << "  if (live) " << out_ptr << "[" << base_expr(N) << "] = " << store_value << ";\n";
+      emit_store("  ");
     }
     o << "}\n";
   }

@@ -35,6 +35,12 @@ struct MapOperandSpec {
 enum class MathPolicy : int { Stored = 0, Folded = 1, Exact = 2 };
 
 struct MapSpec {
+  // Tiled variant (tile_dim >= 0): some inputs ("crossed") are unit-stride along dimension `tile_dim`
+  // while the output is unit-stride along the last one, e.g. out = transpose(x) + y.  A block moves a
+  // 64 x 64 tile of (tile_dim, last dim): crossed inputs are read along tile_dim into LDS and read back
+  // along the last dim, so global loads and stores are both coalesced.  vec is 1.
+  int tile_dim = -1;
+  std::vector<bool> crossed;         // per input; used when tile_dim >= 0
   int rank;                          // rank of the coalesced iteration space (1..kMaxRank)
   int vec;                           // elements per work item: 1, 2, 4 or 8
   int unroll;                        // work items per thread
@@ -46,6 +52,7 @@ struct MapSpec {
 };
 constexpr int kMaxRank = 6;
 constexpr int kMapBlock = 256;
+constexpr int kMapTile = 64;
 
 std::string map_signature(const MapSpec& s);
 std::string map_source(const MapSpec& s);
@@ -69,16 +76,17 @@ enum class ReduceShape { Row, Col };
 
 struct ReduceOperandSpec {
   DType dtype;
-  int axis_stride;  // Row: 0 or 1 (compile time).  Col: -1 = run-time value
+  int axis_stride;        // Row: 0 or 1 (compile time).  Col: -1 = run-time value
+  int inner_stride = -1;  // Col with vec > 1: stride along the lanes' dimension, 0 or 1 (compile time)
 };
 
 struct ReduceSpec {
   ReduceShape shape;
   int outer_rank;                 // 0..3 dims of the output iteration space (coalesced)
-  int vec;                        // Row: elements per load along the axis
+  int vec;                        // Row: elements per load along the axis.  Col: neighbouring outputs per lane
   int threads_per_row;            // Row: T (power of two, 1..1024)
   int block;                      // threads per block
-  int unroll;                     // Row: independent loads in flight per operand
+  int unroll;                     // independent loads in flight per operand
   int waves;                      // Col: waves per block walking the axis
   ReduceOp rop;
   std::vector<ReduceOperandSpec> in;
@@ -87,6 +95,11 @@ struct ReduceSpec {
   Program post;                   // applied once to the folded value; one Load of operand 0 = the folded value
   MathPolicy math_pre = MathPolicy::Folded;
   MathPolicy math_post = MathPolicy::Stored;
+  // A long axis with few outputs is folded in two launches: the first folds S slices of the axis and
+  // stores the f32 accumulators as they are (`raw_out`, no rounding, no post), the second folds those
+  // and finishes as a one-launch reduce would: round to `fold_dtype`, then `post`.
+  bool raw_out = false;
+  DType fold_dtype = DType::F32;  // dtype the folded value is rounded to before `post` (the reduced tensor's)
 };
 
 std::string reduce_signature(const ReduceSpec& s);

@@ -26,14 +26,6 @@ int pow2_ceil(size_t v) {
   return p;
 }
 
-// The iteration space of one kernel seen by all of its operands at once:
-// `shape` plus one stride vector per operand.  Dimensions of size 1 are dropped
-// and neighbouring dimensions are merged when every operand walks them as one.
-struct Space {
-  std::vector<size_t> shape;
-  std::vector<std::vector<size_t>> strides;  // [operand][dim]
-};
-
 Space coalesce(const std::vector<size_t>& shape, const std::vector<std::vector<size_t>>& strides) {
   Space s;
   s.strides.resize(strides.size());
@@ -590,10 +582,29 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   size_t numel = out.layout.numel();
   if (numel == 0) return;
 
+  // The order in which a map visits its elements is free: walk the dimensions in the order of the
+  // OUTPUT's strides (largest first), so that a transposed output written in place is still one
+  // linear sweep and stores are always as coalesced as the layout allows.
+  std::vector<size_t> order;
+  {
+    // dimensions of size 1 stay where they are (their strides mean nothing); the others are sorted
+    std::vector<size_t> real;
+    for (size_t d = 0; d < shape.size(); d++)
+      if (shape[d] != 1) real.push_back(d);
+    std::stable_sort(real.begin(), real.end(), [&](size_t x, size_t y) { return out.layout.strides[x] > out.layout.strides[y]; });
+    size_t next = 0;
+    for (size_t d = 0; d < shape.size(); d++) order.push_back(shape[d] == 1 ? d : real[next++]);
+  }
+  std::vector<size_t> pshape;
+  for (size_t d : order) pshape.push_back(shape[d]);
   std::vector<std::vector<size_t>> strides;
-  for (const TensorData& td : in) strides.push_back(td.layout.strides);
-  strides.push_back(out.layout.strides);
-  Space sp = coalesce(shape, strides);
+  for (size_t k = 0; k <= in.size(); k++) {
+    const std::vector<size_t>& st = k < in.size() ? in[k].layout.strides : out.layout.strides;
+    std::vector<size_t> ps;
+    for (size_t d : order) ps.push_back(st[d]);
+    strides.push_back(ps);
+  }
+  Space sp = coalesce(pshape, strides);
   if (sp.shape.empty()) {
     sp.shape.push_back(1);
     for (auto& s : sp.strides) s.push_back(1);
@@ -630,6 +641,29 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   spec.vec = vec;
   spec.prog = prog;
   spec.math = st_.exact_math ? MathPolicy::Exact : MathPolicy::Stored;
+  // Inputs that run along another dimension than the output (a transposed operand): tiled kernel.
+  if (vec == 1 && R >= 2 && numel >= (size_t(1) << 16) && sp.strides[N - 1][R - 1] == 1 && sp.shape[R - 1] >= 16 &&
+      st_.fusion != FusionMode::Reference) {
+    int ta = -1;
+    for (size_t k = 0; k + 1 < N && ta < 0; k++) {
+      if (sp.strides[k][R - 1] <= 1) continue;
+      for (size_t dd = 0; dd + 1 < R; dd++)
+        if (sp.strides[k][dd] == 1 && sp.shape[dd] >= 16) ta = int(dd);
+    }
+    if (ta >= 0) {
+      size_t ncrossed = 0;
+      for (size_t k = 0; k + 1 < N; k++) {
+        const bool x = sp.strides[k][R - 1] > 1 && sp.strides[k][ta] != 0 && sp.strides[k][ta] < sp.strides[k][R - 1];
+        spec.crossed.push_back(x);
+        ncrossed += x;
+      }
+      if (ncrossed >= 1 && ncrossed <= 3) spec.tile_dim = ta;
+    }
+  }
+  if (spec.tile_dim >= 0) {
+    launch_map_tiled(spec, sp, in, out, in_place);
+    return;
+  }
   const size_t nwork = numel / vec;
   spec.unroll = nwork >= (1u << 20) ? st_.map_unroll : nwork >= (1u << 16) ? 2 : 1;
   size_t bytes = 0;
@@ -675,6 +709,52 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   d << "shape=" << dims(sp.shape) << " vec=" << vec << " unroll=" << spec.unroll << " operands=" << N
     << (in_place ? " in_place" : "");
   r.detail = d.str();
+  record(std::move(r), k, map_pack_args(spec, args));
+}
+
+void Resolver::launch_map_tiled(MapSpec& spec, const Space& sp, const std::vector<TensorData>& in, const TensorData& out,
+                                bool in_place) {
+  const size_t R = sp.shape.size(), N = in.size() + 1, ta = size_t(spec.tile_dim);
+  auto td_of = [&](size_t k) -> const TensorData& { return k < in.size() ? in[k] : out; };
+  spec.unroll = 1;
+  spec.nontemporal = false;
+  for (size_t k = 0; k < N; k++) {
+    MapOperandSpec os;
+    os.dtype = td_of(k).dtype;
+    os.linear = false;
+    os.inner_stride = -1;
+    if (k < in.size()) spec.in.push_back(os);
+    else spec.out = os;
+  }
+  MapArgs args;
+  args.nwork = to_u32(out.layout.numel(), "tensor size");
+  for (size_t d = 0; d < R; d++) args.shape.push_back(to_u32(sp.shape[d], "shape"));
+  for (size_t k = 0; k < N; k++) {
+    const TensorData& td = td_of(k);
+    to_u32(td.layout.extent(), "tensor extent");
+    if (td.layout.extent() * dtype_size(td.dtype) > wkf_buffer_size(td.buffer.get()) + 3)
+      invalid("map kernel: a layout reaches past the end of its buffer");
+    args.ptrs.push_back(element_ptr(td));
+    args.offsets.push_back(to_u32(td.layout.offset, "offset"));
+    std::vector<uint32_t> st;
+    for (size_t d = 0; d < R; d++) st.push_back(to_u32(sp.strides[k][d], "stride"));
+    args.strides.push_back(st);
+  }
+  args.consts = spec.prog.consts;
+  size_t blocks = ((sp.shape[ta] + kMapTile - 1) / kMapTile) * ((sp.shape[R - 1] + kMapTile - 1) / kMapTile);
+  for (size_t d = 0; d + 1 < R; d++)
+    if (d != ta) blocks *= sp.shape[d];
+  std::string sig = map_signature(spec);
+  wkf_kernel* k = kernel(sig, [&] { return map_source(spec); });
+  LaunchRecord r;
+  r.kind = "map";
+  r.signature = sig;
+  r.grid[0] = to_u32(blocks, "grid");
+  r.block[0] = kMapBlock;
+  std::ostringstream d;
+  d << "shape=" << dims(sp.shape) << " tiled dim=" << ta << " operands=" << N << (in_place ? " in_place" : "");
+  r.detail = d.str();
+  r.in_place = in_place;
   record(std::move(r), k, map_pack_args(spec, args));
 }
 
@@ -726,17 +806,116 @@ TensorData Resolver::run_reduce(const NodeP& rn, const std::vector<const Node*>&
   if (axis >= shape.size()) invalid("reduce: axis out of range");
   for (const TensorData& td : eb.operands)
     if (td.layout.shape != shape) invalid("reduce: operand shapes differ");
+
+  ReduceJob job;
+  job.pre = eb.prog;
+  job.operands = eb.operands;
+  job.axis = axis;
+  job.rop = rn->rop;
+  job.post = post;
+  job.fold_dtype = pre_dt;
+
+  // Few outputs over a long axis leave most of the chip idle: fold S slices of the axis side by side
+  // into f32 partials, then fold the partials.  (The reference always uses one workgroup per output,
+  // src/reduce.rs:316-346.)
+  const size_t n = shape[axis];
+  size_t nrows = 1;
+  for (size_t d = 0; d < shape.size(); d++)
+    if (d != axis) nrows *= shape[d];
+  const size_t S = st_.fusion == FusionMode::Reference ? 1 : reduce_split(job, nrows, n);
+  if (S <= 1) return launch_reduce(job);
+
+  // The slice index goes where the axis was when the axis is the unit-stride one (rows and slices then
+  // merge into one dimension), in front otherwise (the lanes stay on the unit-stride outputs).
+  bool row = true;
+  for (const TensorData& td : job.operands) row &= td.layout.strides[axis] <= 1;
+  const size_t pos = row ? axis : 0;
+  ReduceJob first = job;
+  first.raw = true;
+  first.axis = axis + 1;
+  for (TensorData& td : first.operands) {
+    Layout l;
+    l.offset = td.layout.offset;
+    for (size_t d = 0; d < shape.size(); d++) {
+      if (d == pos) {
+        l.shape.push_back(S);
+        l.strides.push_back(td.layout.strides[axis] * (n / S));
+      }
+      l.shape.push_back(d == axis ? n / S : shape[d]);
+      l.strides.push_back(td.layout.strides[d]);
+    }
+    td.layout = l;
+  }
+  if (reduce_outer_rank(first) > 3) return launch_reduce(job);
+  TensorData partial = launch_reduce(first);
+
+  ReduceJob second;
+  {
+    Instr ld;
+    ld.op = Op::Load;
+    ld.dtype = DType::F32;
+    ld.operand = 0;
+    second.pre.ins.push_back(ld);
+    second.pre.result = 0;
+  }
+  second.operands = {partial};
+  second.axis = pos;
+  second.rop = rn->rop;
+  second.post = post;
+  second.fold_dtype = pre_dt;
+  return launch_reduce(second);
+}
+
+size_t Resolver::reduce_outer_rank(const ReduceJob& job) {
+  const std::vector<size_t>& shape = job.operands[0].layout.shape;
+  std::vector<size_t> out_shape;
+  std::vector<std::vector<size_t>> ostr(job.operands.size() + 1);
+  for (size_t d = 0; d < shape.size(); d++) {
+    if (d == job.axis) continue;
+    out_shape.push_back(shape[d]);
+    for (size_t k = 0; k < job.operands.size(); k++) ostr[k].push_back(job.operands[k].layout.strides[d]);
+  }
+  ostr.back() = Layout::contiguous_strides(out_shape);
+  return coalesce(out_shape, ostr).shape.size();
+}
+
+size_t Resolver::reduce_split(const ReduceJob& job, size_t nrows, size_t n) {
+  if (nrows == 0 || n < 4096) return 1;
+  bool row = true;
+  for (const TensorData& td : job.operands) row &= td.layout.strides[job.axis] <= 1;
+  wkf_props props;
+  check(wkf_device_props(dev_, &props));
+  const size_t cus = size_t(std::max(1, props.compute_units));
+  size_t S = 1;
+  if (row) {
+    // one block of 1024 lanes per row: split until there are about four blocks per compute unit,
+    // keeping at least 8192 elements per slice
+    while (nrows * S < 4 * cus && n / (2 * S) >= 8192 && n % (2 * S) == 0) S *= 2;
+  } else {
+    // one block of 16 waves per 256 (at best) neighbouring outputs: keep at least 128 axis steps per slice
+    const size_t blocks = (nrows + 255) / 256;
+    while (blocks * S < 8 * cus && n / (2 * S) >= 128 && n % (2 * S) == 0) S *= 2;
+  }
+  return S;
+}
+
+TensorData Resolver::launch_reduce(const ReduceJob& job) {
+  const std::vector<TensorData>& ops = job.operands;
+  const std::vector<size_t>& shape = ops[0].layout.shape;
+  const size_t axis = job.axis;
+  const DType pre_dt = job.pre.result_dtype();
+  const DType out_dt = job.raw ? DType::F32 : job.post.result_dtype();
   std::vector<size_t> out_shape;
   for (size_t d = 0; d < shape.size(); d++)
     if (d != axis) out_shape.push_back(shape[d]);
-  TensorData out = alloc(out_shape, post.result_dtype(), false);
+  TensorData out = alloc(out_shape, out_dt, false);
   const size_t nrows = out.layout.numel();
   const size_t n = shape[axis];
   if (nrows == 0) return out;
 
-  const size_t N = eb.operands.size();
+  const size_t N = ops.size();
   std::vector<std::vector<size_t>> ostr;
-  for (const TensorData& td : eb.operands) {
+  for (const TensorData& td : ops) {
     std::vector<size_t> s;
     for (size_t d = 0; d < shape.size(); d++)
       if (d != axis) s.push_back(td.layout.strides[d]);
@@ -749,10 +928,12 @@ TensorData Resolver::run_reduce(const NodeP& rn, const std::vector<const Node*>&
 
   ReduceSpec spec;
   spec.outer_rank = int(Ro);
-  spec.rop = rn->rop;
-  spec.out_dtype = post.result_dtype();
-  spec.pre = eb.prog;
-  spec.post = post;
+  spec.rop = job.rop;
+  spec.out_dtype = out_dt;
+  spec.pre = job.pre;
+  spec.post = job.post;
+  spec.raw_out = job.raw;
+  spec.fold_dtype = job.fold_dtype;
   spec.math_pre = st_.exact_math ? MathPolicy::Exact : MathPolicy::Folded;
   spec.math_post = st_.exact_math ? MathPolicy::Exact : MathPolicy::Stored;
   spec.vec = 1;
@@ -761,19 +942,21 @@ TensorData Resolver::run_reduce(const NodeP& rn, const std::vector<const Node*>&
   spec.unroll = 1;
   spec.waves = 1;
   bool row = true;
-  for (const TensorData& td : eb.operands) row &= (n <= 1 || td.layout.strides[axis] <= 1);
+  for (const TensorData& td : ops) row &= (n <= 1 || td.layout.strides[axis] <= 1);
   spec.shape = row ? ReduceShape::Row : ReduceShape::Col;
+
+  size_t max_elem = 2;
+  for (const TensorData& td : ops) max_elem = std::max(max_elem, dtype_size(td.dtype));
+  max_elem = std::max(max_elem, dtype_size(out_dt));
 
   LaunchRecord r;
   std::ostringstream d;
   if (row) {
-    size_t max_elem = 2;
-    for (const TensorData& td : eb.operands) max_elem = std::max(max_elem, dtype_size(td.dtype));
     int vec = int(16 / max_elem);
     auto vec_ok = [&](int V) {
       if (n % V) return false;
       for (size_t k = 0; k < N; k++) {
-        const TensorData& td = eb.operands[k];
+        const TensorData& td = ops[k];
         if (td.layout.strides[axis] == 0) continue;
         if (td.layout.offset % V) return false;
         for (size_t dd = 0; dd < Ro; dd++)
@@ -794,30 +977,55 @@ TensorData Resolver::run_reduce(const NodeP& rn, const std::vector<const Node*>&
     spec.block = std::max(256, T);
     size_t per_lane = (nvec + T - 1) / T;
     spec.unroll = per_lane >= 4 ? 4 : per_lane >= 2 ? 2 : 1;
-    for (const TensorData& td : eb.operands)
-      spec.in.push_back({td.dtype, (n <= 1 || td.layout.strides[axis] == 0) ? 0 : 1});
+    for (const TensorData& td : ops) spec.in.push_back({td.dtype, (n <= 1 || td.layout.strides[axis] == 0) ? 0 : 1, -1});
     size_t rpb = size_t(spec.block / T);
     r.grid[0] = to_u32((nrows + rpb - 1) / rpb, "grid");
     r.block[0] = uint32_t(spec.block);
     r.kind = "red_row";
     d << "rows=" << nrows << " n=" << n << " vec=" << vec << " threads_per_row=" << T << " unroll=" << spec.unroll;
   } else {
+    // Lanes sit on the last outer dim; V neighbouring outputs per lane when every operand is
+    // unit-stride (or a broadcast) and 16-byte aligned there.
+    const size_t lanes_dim = Ro ? sp.shape[Ro - 1] : 1;
+    int vec = Ro ? int(16 / max_elem) : 1;
+    auto vec_ok = [&](int V) {
+      if (lanes_dim % V) return false;
+      for (size_t k = 0; k <= N; k++) {
+        const TensorData& td = k < N ? ops[k] : out;
+        const size_t inner = sp.strides[k][Ro - 1];
+        if (inner > 1) return false;
+        if (inner == 0) {
+          if (k == N) return false;
+          continue;
+        }
+        if (td.layout.offset % V) return false;
+        for (size_t dd = 0; dd + 1 < Ro; dd++)
+          if (sp.strides[k][dd] % V) return false;
+        if (k < N && td.layout.strides[axis] % V) return false;
+      }
+      return true;
+    };
+    while (vec > 1 && !vec_ok(vec)) vec /= 2;
+    spec.vec = vec;
     spec.waves = n >= 64 ? 16 : n >= 8 ? 4 : 1;
-    for (const TensorData& td : eb.operands) spec.in.push_back({td.dtype, -1});
-    size_t lanes_dim = Ro ? sp.shape[Ro - 1] : 1;
-    size_t rest = nrows / lanes_dim;
-    r.grid[0] = to_u32(((lanes_dim + 63) / 64) * rest, "grid");
+    const size_t steps = (n + spec.waves - 1) / spec.waves;
+    spec.unroll = steps >= 4 ? 4 : steps >= 2 ? 2 : 1;
+    for (size_t k = 0; k < N; k++) spec.in.push_back({ops[k].dtype, -1, vec > 1 ? int(sp.strides[k][Ro - 1]) : -1});
+    const size_t per_block = size_t(64) * vec;
+    const size_t rest = nrows / lanes_dim;
+    r.grid[0] = to_u32(((lanes_dim + per_block - 1) / per_block) * rest, "grid");
     r.block[0] = uint32_t(64 * spec.waves);
     r.kind = "red_col";
-    d << "outputs=" << nrows << " n=" << n << " waves=" << spec.waves;
+    d << "outputs=" << nrows << " n=" << n << " vec=" << vec << " waves=" << spec.waves << " unroll=" << spec.unroll;
   }
+  if (job.raw) d << " partial";
 
   ReduceArgs args;
   args.nrows = to_u32(nrows, "output size");
   args.n = to_u32(n, "axis length");
   for (size_t dd = 0; dd < Ro; dd++) args.oshape.push_back(to_u32(sp.shape[dd], "shape"));
   for (size_t k = 0; k <= N; k++) {
-    const TensorData& td = k < N ? eb.operands[k] : out;
+    const TensorData& td = k < N ? ops[k] : out;
     to_u32(td.layout.extent(), "tensor extent");
     args.ptrs.push_back(element_ptr(td));
     args.offsets.push_back(to_u32(td.layout.offset, "offset"));
@@ -826,14 +1034,15 @@ TensorData Resolver::run_reduce(const NodeP& rn, const std::vector<const Node*>&
     args.ostrides.push_back(st);
     if (k < N) args.astrides.push_back(to_u32(td.layout.strides[axis], "stride"));
   }
-  args.consts = eb.prog.consts;
-  args.consts.insert(args.consts.end(), post.consts.begin(), post.consts.end());
+  args.consts = job.pre.consts;
+  if (!job.raw) args.consts.insert(args.consts.end(), job.post.consts.begin(), job.post.consts.end());
 
   std::string sig = reduce_signature(spec);
   wkf_kernel* k = kernel(sig, [&] { return reduce_source(spec); });
   r.signature = sig;
   r.detail = d.str();
   record(std::move(r), k, reduce_pack_args(spec, args));
+  (void)pre_dt;
   return out;
 }
 

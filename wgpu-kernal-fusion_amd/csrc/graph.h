@@ -35,6 +35,14 @@ struct Settings {
   size_t nontemporal_bytes = size_t(32) << 20;  // map kernels moving at least this much use streaming loads/stores
 };
 
+// The iteration space of one kernel seen by all of its operands at once:
+// `shape` plus one stride vector per operand.  Dimensions of size 1 are dropped
+// and neighbouring dimensions are merged when every operand walks them as one.
+struct Space {
+  std::vector<size_t> shape;
+  std::vector<std::vector<size_t>> strides;  // [operand][dim]
+};
+
 class Resolver {
  public:
   Resolver(wkf_device* dev, const Settings& st, std::vector<LaunchRecord>* log) : dev_(dev), st_(st), log_(log) {}
@@ -74,6 +82,20 @@ class Resolver {
   bool try_row_kernel(const NodeP& root, TensorData* out);
   int row_build(RowBuild& rb, Program& prog, std::map<const Node*, int>& memo, std::map<int, int>& loads, const NodeP& n);
   TensorData run_reduce(const NodeP& reduce, const std::vector<const Node*>& post_chain);
+  // One reduce launch: fold `pre(operands)` over `axis`, then (unless `raw`) round to `fold_dtype` and apply `post`.
+  struct ReduceJob {
+    Program pre, post;
+    std::vector<TensorData> operands;  // all of one shape
+    size_t axis = 0;
+    ReduceOp rop = ReduceOp::Sum;
+    DType fold_dtype = DType::F32;
+    bool raw = false;                  // store the f32 accumulators (first launch of a split reduce)
+  };
+  TensorData launch_reduce(const ReduceJob& job);
+  // Number of axis slices a reduce is split into (1 = one launch).
+  size_t reduce_split(const ReduceJob& job, size_t nrows, size_t n);
+  // Rank of the job's output iteration space after merging dimensions (the kernels take up to 3).
+  size_t reduce_outer_rank(const ReduceJob& job);
   TensorData run_matmul(const NodeP& n);
   TensorData run_map_layout(const NodeP& n);
   TensorData run_resize(const NodeP& n);
@@ -81,6 +103,7 @@ class Resolver {
 
   // out[i] = prog(operands[i]) over out.layout.shape; every operand layout has that shape.
   void launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
+  void launch_map_tiled(MapSpec& spec, const Space& sp, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
   TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero);
   TensorData make_contiguous(const TensorData& td);
   void record(LaunchRecord&& r, wkf_kernel* k, const std::vector<unsigned char>& args);
