@@ -137,6 +137,12 @@ int wkf_tensor_materialize(wkf_tensor* t);
 int wkf_tensor_kernel_count(const wkf_tensor* t);
 int wkf_tensor_kernel_info(const wkf_tensor* t, int i, uint64_t* elapsed_ns, char* kind, size_t kind_cap,
                            char* signature, size_t signature_cap, char* detail, size_t detail_cap);
+/* Tensor::graphvis, src/tensor.rs:641-643 -> src/compute_graph/visualize.rs:13-271: the lazy graph below `t`
+ * as Graphviz DOT text (`digraph "ComputeGraph"`), one node per graph node labelled
+ * `<name> ([shape] dtype) #<id>` and one edge per input, in the reference's format.  Writes at most `cap`
+ * bytes (NUL-terminated) and the full length + 1 into *needed.  Materialising does not change the graph
+ * (nor does it in the reference: ComputeGraph::resolve keeps every node, src/compute_graph/mod.rs:241-248). */
+int wkf_tensor_graphvis(const wkf_tensor* t, char* out, size_t cap, size_t* needed);
 /* The generated HIP source of a kernel signature seen by this process (for inspection and tests). */
 int wkf_kernel_source(const char* signature, char* out, size_t cap, size_t* needed);
 

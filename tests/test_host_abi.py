@@ -120,6 +120,27 @@ def test_hiprtc_failure_is_reported_with_the_log(wkf, planner):
     assert "hiprtc" in msg and "error" in msg
 
 
+def test_graphvis_is_the_reference_dot_format(wkf, planner):
+    # node ids `<name> ([shape] dtype) #<n>`, edges input -> consumer, shared nodes once (src/compute_graph/visualize.rs:13-271)
+    x = wkf.Tensor.new(planner, np.ones((3, 2), dtype=np.float32))
+    y = wkf.Tensor.new(planner, np.ones((3, 2), dtype=np.float16))
+    m = x * 2.0
+    t = (m + m.exp()).cast(wkf.F16).transpose(0, 1).mat_mul(y).sum(1)
+    dot = t.graphvis()
+    lines = [l.strip() for l in dot.strip().splitlines()]
+    assert lines[0] == 'digraph "ComputeGraph" {' and lines[-1] == "}"
+    nodes = [l for l in lines[1:-1] if "->" not in l]
+    edges = [l for l in lines[1:-1] if "->" in l]
+    names = [n.split(" (")[0].strip('"') for n in nodes]
+    assert names == ["tensor", "multiply_const", "exp", "add", "cast", "slice", "tensor", "matmul", "sum"]
+    assert '"slice ([2, 3] f16) #5";' in nodes and '"matmul ([2, 2] f16) #7";' in nodes and '"sum ([2] f16) #8";' in nodes
+    assert len(edges) == 9  # multiply_const feeds both exp and add and is listed once
+    assert '"multiply_const ([3, 2] f32) #1" -> "exp ([3, 2] f32) #2";' in edges
+    assert '"multiply_const ([3, 2] f32) #1" -> "add ([3, 2] f32) #3";' in edges
+    t.materialize()
+    assert t.graphvis() == dot  # resolving keeps the graph (src/compute_graph/mod.rs:241-248)
+
+
 def test_arange_is_a_host_loop(wkf, planner):
     assert np.array_equal(wkf.Tensor.arange(planner, 0.0, 10.0).to_numpy(), np.arange(10, dtype=np.float32))
     assert np.array_equal(wkf.Tensor.arange_step(planner, 0.0, 10.0, 2.0).to_numpy(), np.array([0, 2, 4, 6, 8], dtype=np.float32))

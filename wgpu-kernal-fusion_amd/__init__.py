@@ -46,7 +46,7 @@ EXPORTS = [
     "wkf_tensor_reshape", "wkf_tensor_unsqueeze", "wkf_tensor_slice_assign", "wkf_tensor_cat", "wkf_tensor_silu",
     "wkf_tensor_layer_norm", "wkf_tensor_rope", "wkf_tensor_softmax", "wkf_tensor_softmax_last_dim",
     "wkf_tensor_arange", "wkf_tensor_materialize", "wkf_tensor_kernel_count", "wkf_tensor_kernel_info",
-    "wkf_kernel_source", "wkf_tensor_as_slice", "wkf_slice_free", "wkf_slice_rank", "wkf_slice_dtype",
+    "wkf_kernel_source", "wkf_tensor_graphvis", "wkf_tensor_as_slice", "wkf_slice_free", "wkf_slice_rank", "wkf_slice_dtype",
     "wkf_slice_layout", "wkf_slice_data", "wkf_slice_get",
 ]
 
@@ -119,6 +119,7 @@ def load():
     lib.wkf_tensor_kernel_info.argtypes = [c_void_p, c_int, POINTER(c_uint64), c_char_p, c_size_t, c_char_p, c_size_t,
                                            c_char_p, c_size_t]
     lib.wkf_kernel_source.argtypes = [c_char_p, c_char_p, c_size_t, POINTER(c_size_t)]
+    lib.wkf_tensor_graphvis.argtypes = [c_void_p, c_char_p, c_size_t, POINTER(c_size_t)]
     lib.wkf_tensor_as_slice.argtypes = [c_void_p, POINTER(c_void_p)]
     lib.wkf_slice_free.argtypes = [c_void_p]
     lib.wkf_slice_free.restype = None
@@ -533,6 +534,14 @@ class Tensor:
 
     def to_numpy(self):
         return self.as_slice().to_numpy()
+
+    def graphvis(self):
+        """Tensor::graphvis (src/tensor.rs:641-643 of the reference): the lazy graph below this tensor as DOT text."""
+        need = c_size_t()
+        _check(self._lib.wkf_tensor_graphvis(self._h, None, 0, byref(need)))
+        buf = ctypes.create_string_buffer(need.value)
+        _check(self._lib.wkf_tensor_graphvis(self._h, buf, need.value, byref(need)))
+        return buf.value.decode()
 
     def kernels(self):
         """Kernels launched by the last materialize / as_slice, with GPU times."""

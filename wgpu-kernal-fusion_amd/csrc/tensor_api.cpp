@@ -750,6 +750,59 @@ int wkf_kernel_source(const char* signature, char* out, size_t cap, size_t* need
   });
 }
 
+extern "C++" {
+namespace {
+// DOT text of the lazy graph below `root` in the reference's format (src/compute_graph/visualize.rs:13-271):
+// one node per graph node, labelled `<name> ([shape] dtype) #<id>`, edges from inputs to their consumer, a
+// node reached twice emitted once.  Every layout op is called "slice" there (visualize.rs:196).
+std::string graph_dot(const NodeP& root) {
+  std::ostringstream o;
+  o << "digraph \"ComputeGraph\" {\n";
+  std::map<const Node*, std::string> ids;
+  std::function<std::string(const NodeP&)> visit = [&](const NodeP& n) -> std::string {
+    auto it = ids.find(n.get());
+    if (it != ids.end()) return it->second;
+    std::vector<std::string> inputs;
+    if (n->kind != NodeKind::Tensor) {
+      if (n->a) inputs.push_back(visit(n->a));
+      if (n->b) inputs.push_back(visit(n->b));
+    }
+    const char* name = "tensor";
+    switch (n->kind) {
+      case NodeKind::Tensor: name = "tensor"; break;
+      case NodeKind::ElementWise:
+      case NodeKind::PairWise: name = op_name(n->op); break;
+      case NodeKind::Reduce: name = reduce_name(n->rop); break;
+      case NodeKind::MatMul: name = "matmul"; break;
+      case NodeKind::MapLayout: name = "slice"; break;
+      case NodeKind::Resize: name = "resize"; break;
+      case NodeKind::SliceAssign: name = "slice_assign"; break;
+    }
+    std::ostringstream id;
+    id << '"' << name << " ([";
+    for (size_t d = 0; d < n->shape.size(); d++) id << (d ? ", " : "") << n->shape[d];
+    id << "] " << dtype_name(n->dtype) << ") #" << ids.size() << '"';
+    ids[n.get()] = id.str();
+    o << "  " << id.str() << ";\n";
+    for (const std::string& in : inputs) o << "  " << in << " -> " << id.str() << ";\n";
+    return id.str();
+  };
+  visit(root);
+  o << "}\n";
+  return o.str();
+}
+}  // namespace
+}  // extern "C++"
+
+int wkf_tensor_graphvis(const wkf_tensor* t, char* out, size_t cap, size_t* needed) {
+  return guarded([&] {
+    need(t, "wkf_tensor_graphvis");
+    const std::string dot = graph_dot(t->node);
+    if (needed) *needed = dot.size() + 1;
+    copy_str(dot, out, cap);
+  });
+}
+
 int wkf_tensor_as_slice(wkf_tensor* t, wkf_slice** out) {
   return guarded([&] {
     need(t, "wkf_tensor_as_slice");
