@@ -129,7 +129,8 @@ def summarise(wl, kernels, wall_s, steps, batch_us):
             "kernels": kernels, "gpu_us_per_step": round(gpu_us, 2),
             "achieved": round(wl.work / gpu_us * scale, 1), "peak": wl.peak,
             "frac": round(wl.work / gpu_us * scale / wl.peak, 4), "batch_us_per_step": batch_us,
-            "batch_achieved": round(wl.work / batch_us * scale, 1), "batch_frac": round(wl.work / batch_us * scale / wl.peak, 4),
+            "batch_achieved": round(wl.work / batch_us * scale, 1) if batch_us else None,
+            "batch_frac": round(wl.work / batch_us * scale / wl.peak, 4) if batch_us else None,
             "wall_ms_per_step": round(wall_s / steps * 1e3, 4),
             "wall_rate": round(wl.work * steps / wall_s * (1e-9 if wl.unit == "GB/s" else 1e-12), 1)}
 
@@ -211,6 +212,32 @@ def cpu_baseline(seeded):
                       "oracle/port.c with OpenMP (the reference's wgpu path cannot run: no Rust toolchain, no Vulkan ICD)"}
 
 
+def plan_only(w):
+    """Plans (and so JIT-compiles for gfx950) every kernel this benchmark launches, at the benchmark's shapes, on a
+    device that has no GPU behind it.  Nothing is computed or timed; the inputs are zeros."""
+    dev = w.Device.planner()
+
+    def zeros(config, tensor, shape, dist, dtype=np.float32, **kw):
+        return np.zeros(shape, dtype=dtype)
+
+    before = dev.module_stats()
+    copy = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32)).reshape([1 << 14, 1 << 14])
+    copy.materialize()
+    del copy
+    for gname in ("c1", "c2", "c3", "c4", "c5"):
+        wls = build_workloads(w, dev, zeros, {gname})
+        for one in wls.values():
+            for mode in ((w.FUSION_TREE, w.FUSION_REFERENCE) if gname in ("c3", "c4") else (w.FUSION_TREE,)):
+                dev.set_fusion(mode)
+                for t in one.variants[0]:
+                    t.materialize()
+            dev.set_fusion(w.FUSION_TREE)
+        del wls
+    after = dev.module_stats()
+    print(json.dumps({"plan_only": True, "kernels_compiled": after["compiled"] - before["compiled"],
+                      "kernels_from_disk_cache": after["disk_hits"] - before["disk_hits"]}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -219,6 +246,8 @@ def main():
     ap.add_argument("--no-detail", action="store_true", help="only the headline configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5 for the detail table")
+    ap.add_argument("--plan-only", action="store_true",
+                    help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every kernel, no collectives); --gpus must be 1. "
@@ -229,6 +258,9 @@ def main():
     datagen = importlib.util.module_from_spec(dg_spec)
     dg_spec.loader.exec_module(datagen)
     seeded = datagen.seeded
+    if args.plan_only:
+        plan_only(w)
+        return
     dev = w.Device.new(0)
     props = dev.props()
     if args.only == "copy":
@@ -287,6 +319,18 @@ def main():
                 wall_s = measure_wall(dev, one, steps, 5)
                 batch_us = round(measure_batch(w, dev, one, steps, 5), 2)
                 detail.append(summarise(one, ks, wall_s, steps, batch_us))
+                if gname in ("c3", "c4"):
+                    # the same graph under the reference's own fusion rules (its kernel decomposition):
+                    # same algorithmic work, more passes over memory
+                    dev.set_fusion(w.FUSION_REFERENCE)
+                    try:
+                        ks = measure_kernels(dev, one, steps, 5)
+                        wall_s = measure_wall(dev, one, steps, 5)
+                        row = summarise(one, ks, wall_s, steps, None)
+                        row["name"] += " -- reference kernel decomposition"
+                        detail.append(row)
+                    finally:
+                        dev.set_fusion(w.FUSION_TREE)
             del wls
             dev.trim()
         result["all_configs"] = detail
