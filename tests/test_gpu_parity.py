@@ -323,6 +323,35 @@ def test_resize_reshape_slice_assign_cat_are_bit_exact(gpu):
         assert_ulp(g, w.to_numpy(), 0, f"copy {i}")
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+def test_consumers_of_cat_run_per_piece(gpu, dtype):
+    # an element-wise consumer of cat([A, B]) never copies the pieces together: one kernel with two stores
+    # when the pieces have one shape, two kernels otherwise; cats below broadcasts / narrows are cut the same way
+    api = HipAPI(gpu)
+    a, a2 = data((7, 4), -2, 2, dtype, 31), data((7, 4), -2, 2, dtype, 32)
+    b = data((7, 6), -2, 2, dtype, 33)
+    c8, c10 = data((7, 8), -2, 2, dtype, 34), data((7, 10), -2, 2, dtype, 35)
+    t = data((5, 4), -2, 2, dtype, 36)
+    x = data((3, 5, 8), -2, 2, dtype, 37)
+
+    def progs(T, a, a2, b, c8, c10, t, x):
+        table = T.cat([t, t * 2.0], 1).narrow(0, 1, 3)                     # [3, 8], cut at column 4
+        xs = x.narrow(1, 1, 3)                                              # [3, 3, 8]
+        return [T.cat([a, a2], 1) * c8 + 1.0,                              # equal pieces
+                T.cat([a, b], 1) * c10,                                    # unequal pieces
+                (T.cat([a.exp(), -a2], 1) - c8) * T.cat([a2, a], 1),       # two cats at the same seam
+                T.cat([xs.narrow(2, 4, 4), xs.narrow(2, 0, 4)], 2) * table.broadcast([3, 3, 8]) + xs,
+                T.cat([a, a2], 0) + T.cat([a2, a], 0),                     # cut along dim 0
+                (T.cat([a, a2], 1) * c8).sum(1)]                           # a reduce consumer takes the ordinary path
+
+    got = hip_values_many(progs(api.T, *[api.tensor(v) for v in (a, a2, b, c8, c10, t, x)]))
+    want = progs(OTensor, *[OTensor(v) for v in (a, a2, b, c8, c10, t, x)])
+    for i, (g, w) in enumerate(zip(got[:5], want[:5])):
+        assert_ulp(g, w.to_numpy(), 2 if i == 2 else 0, f"cat consumer {i}")
+    assert np.allclose(got[5].astype(np.float64), want[5].to_numpy().astype(np.float64), rtol=1e-5 if dtype == np.float32 else 1e-2,
+                       atol=1e-5 if dtype == np.float32 else 2e-2)
+
+
 def test_slice_assign_does_not_change_a_tensor_the_caller_holds(gpu, wkf):
     base = np.zeros((4, 4), dtype=np.float32)
     leaf = wkf.Tensor.new(gpu, base)

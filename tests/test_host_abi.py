@@ -237,8 +237,14 @@ def test_tree_mode_fuses_pair_wise_trees_and_copies(wkf, planner):
     assert _kinds(_x(wkf, planner, (8, 30)).softmax_last_dim()) == ["red_row", "red_row", "map"]
     q = _x(wkf, planner, (2, 8, 16))
     cos, sin = _x(wkf, planner, (8, 8), seed=4), _x(wkf, planner, (8, 8), seed=5)
-    kinds = _kinds(q.rope(cos, sin))
-    assert all(k == "map" for k in kinds) and len(kinds) <= 8
+    # rope = ONE kernel: the cats of rotate_half and of the duplicated tables are cut at the seam, both halves of the
+    # result are stored by the same kernel, and x1, x2, cos, sin are each loaded once (the reference: about 10 kernels)
+    r = q.rope(cos, sin)
+    assert _kinds(r) == ["map"]
+    assert "outputs=2" in r.kernels()[0].detail and "operands=6" in r.kernels()[0].detail
+    # pieces of different widths: one kernel per piece
+    odd = _x(wkf, planner, (2, 8, 10)).narrow(2, 0, 3)
+    assert _kinds(wkf.Tensor.cat([odd, _x(wkf, planner, (2, 8, 5), seed=6)], 2) * _x(wkf, planner, (2, 8, 8), seed=7)) == ["map", "map"]
 
 
 def test_few_outputs_over_a_long_axis_fold_in_two_launches(wkf, planner):

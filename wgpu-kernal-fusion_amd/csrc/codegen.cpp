@@ -174,6 +174,9 @@ std::string map_signature(const MapSpec& s) {
   for (const auto& i : s.in) o << dtype_name(i.dtype) << (i.linear ? 'L' : 'S') << i.inner_stride << ',';
   o << "|out:" << dtype_name(s.out.dtype) << (s.out.linear ? 'L' : 'S') << s.out.inner_stride;
   o << "|m" << int(s.math) << "|" << s.prog.signature();
+  for (size_t j = 0; j < s.more_out.size(); j++)
+    o << "|out+:" << dtype_name(s.more_out[j].dtype) << (s.more_out[j].linear ? 'L' : 'S') << s.more_out[j].inner_stride << "|"
+      << s.more_prog[j].signature();
   if (s.tile_dim >= 0) {
     o << "|tile" << s.tile_dim << ':';
     for (size_t k = 0; k < s.in.size(); k++) o << (s.crossed[k] ? 'x' : '-');
@@ -267,23 +270,45 @@ std::string map_tiled_source(const MapSpec& s) {
 
 std::string map_source(const MapSpec& s) {
   if (s.tile_dim >= 0) return map_tiled_source(s);
-  const int N = int(s.in.size()) + 1;  // operands incl. out
+  const int NI = int(s.in.size());
+  const int NO = 1 + int(s.more_out.size());
+  const int N = NI + NO;  // operands: inputs, then outputs
   const int R = s.rank, V = s.vec, U = s.unroll;
-  const int NC = s.prog.consts.empty() ? 1 : int(s.prog.consts.size());
+  std::vector<const Program*> progs = {&s.prog};
+  std::vector<const MapOperandSpec*> outs = {&s.out};
+  for (int j = 1; j < NO; j++) {
+    progs.push_back(&s.more_prog[j - 1]);
+    outs.push_back(&s.more_out[j - 1]);
+  }
+  std::vector<int> coff;  // where each program's constants start in the argument block
+  int NC = 0;
+  for (const Program* p : progs) {
+    coff.push_back(NC);
+    NC += int(p->consts.size());
+  }
+  NC = std::max(1, NC);
   std::ostringstream o;
   o << kPrelude;
-  if (uses_math(s.prog, s.math)) o << kMath;
+  bool any_math = false, any_trig = false;
+  std::vector<bool> trig;
+  for (const Program* p : progs) {
+    any_math |= uses_math(*p, s.math);
+    trig.push_back(uses_trig(*p, s.math));
+    any_trig |= trig.back();
+  }
+  if (any_math) o << kMath;
   o << "struct Args { void* p[" << N << "]; u32 nwork; u32 shape[" << R << "]; u32 off[" << N << "]; u32 stride[" << N
     << "][" << R << "]; float c[" << NC << "]; };\n";
   std::vector<DType> types;
   for (const auto& i : s.in) types.push_back(i.dtype);
-  emit_program(o, s.prog, "wkf_expr", types, s.math);
+  auto fn = [&](int q) { return q == 0 ? std::string("wkf_expr") : "wkf_expr" + std::to_string(q); };
+  for (int q = 0; q < NO; q++) emit_program(o, *progs[q], fn(q), types, s.math);
 
   bool need_unravel = false;
   for (const auto& i : s.in) need_unravel |= !i.linear;
-  need_unravel |= !s.out.linear;
+  for (const MapOperandSpec* op : outs) need_unravel |= !op->linear;
 
-  auto operand = [&](int k) -> const MapOperandSpec& { return k < N - 1 ? s.in[k] : s.out; };
+  auto operand = [&](int k) -> const MapOperandSpec& { return k < NI ? s.in[k] : *outs[k - NI]; };
   auto index_expr = [&](int k, int j) {
     const MapOperandSpec& op = operand(k);
     std::ostringstream e;
@@ -313,7 +338,7 @@ std::string map_source(const MapSpec& s) {
     }
   };
   auto emit_loads = [&](int j, const char* ind) {
-    for (int k = 0; k < N - 1; k++) {
+    for (int k = 0; k < NI; k++) {
       const MapOperandSpec& op = s.in[k];
       std::string ptr = std::string("((const ") + ctype(op.dtype) + "*)a.p[" + std::to_string(k) + "])";
       if (is_vec_load(k)) {
@@ -329,40 +354,50 @@ std::string map_source(const MapSpec& s) {
       }
     }
   };
-  const bool trig = uses_trig(s.prog, s.math);
-  const std::string ot = vtype(s.out.dtype, V);
-  const std::string optr = std::string("((") + ctype(s.out.dtype) + "*)a.p[" + std::to_string(N - 1) + "])";
+  // value name of output q, work item j
+  auto oname = [&](int q, int j) { return "o" + std::to_string(j) + (q ? "_" + std::to_string(q) : ""); };
   auto emit_compute = [&](int j, const char* ind, bool far_variant) {
-    for (int e = 0; e < V; e++) {
-      o << ind << "o" << j;
-      if (V > 1) o << "[" << e << "]";
-      o << " = wkf_expr" << (far_variant ? "_far" : "") << "(";
-      for (int k = 0; k < N - 1; k++) {
-        o << "r" << k << "_" << j;
-        if (is_vec_load(k)) o << "[" << e << "]";
-        o << ", ";
+    for (int q = 0; q < NO; q++) {
+      if (far_variant && !trig[q]) continue;
+      for (int e = 0; e < V; e++) {
+        o << ind << oname(q, j);
+        if (V > 1) o << "[" << e << "]";
+        o << " = " << fn(q) << (far_variant ? "_far" : "") << "(";
+        for (int k = 0; k < NI; k++) {
+          o << "r" << k << "_" << j;
+          if (is_vec_load(k)) o << "[" << e << "]";
+          o << ", ";
+        }
+        o << "a.c";
+        if (coff[q]) o << " + " << coff[q];
+        o << (trig[q] && !far_variant ? ", far" : "") << ");\n";
       }
-      o << "a.c" << (trig && !far_variant ? ", far" : "") << ");\n";
     }
   };
   auto emit_store = [&](int j, const char* ind) {
-    if (V > 1) {
-      if (s.nontemporal && s.out.linear)
-        o << ind << "__builtin_nontemporal_store(o" << j << ", (" << ot << "*)(" << optr << " + (" << index_expr(N - 1, j)
-          << ")));\n";
-      else
-        o << ind << "*(" << ot << "*)(" << optr << " + (" << index_expr(N - 1, j) << ")) = o" << j << ";\n";
-    } else {
-      o << ind << optr << "[" << index_expr(N - 1, j) << "] = o" << j << ";\n";
+    for (int q = 0; q < NO; q++) {
+      const MapOperandSpec& op = *outs[q];
+      const std::string ot = vtype(op.dtype, V);
+      const std::string optr = std::string("((") + ctype(op.dtype) + "*)a.p[" + std::to_string(NI + q) + "])";
+      if (V > 1) {
+        if (s.nontemporal && op.linear)
+          o << ind << "__builtin_nontemporal_store(" << oname(q, j) << ", (" << ot << "*)(" << optr << " + (" << index_expr(NI + q, j)
+            << ")));\n";
+        else
+          o << ind << "*(" << ot << "*)(" << optr << " + (" << index_expr(NI + q, j) << ")) = " << oname(q, j) << ";\n";
+      } else {
+        o << ind << optr << "[" << index_expr(NI + q, j) << "] = " << oname(q, j) << ";\n";
+      }
     }
   };
   // loads -> fused expression on every element -> (rarely) redo through the far variant -> stores
   auto emit_batch = [&](int j0, int j1, const std::string& ind) {
     for (int j = j0; j < j1; j++) emit_loads(j, ind.c_str());
-    for (int j = j0; j < j1; j++) o << ind << ot << " o" << j << ";\n";
-    if (trig) o << ind << "bool far = false;\n";
+    for (int j = j0; j < j1; j++)
+      for (int q = 0; q < NO; q++) o << ind << vtype(outs[q]->dtype, V) << " " << oname(q, j) << ";\n";
+    if (any_trig) o << ind << "bool far = false;\n";
     for (int j = j0; j < j1; j++) emit_compute(j, ind.c_str(), false);
-    if (trig) {
+    if (any_trig) {
       o << ind << "if (__builtin_expect(far, 0)) {\n";
       for (int j = j0; j < j1; j++) emit_compute(j, (ind + "  ").c_str(), true);
       o << ind << "}\n";
@@ -391,7 +426,7 @@ std::string map_source(const MapSpec& s) {
 }
 
 std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a) {
-  const size_t N = s.in.size() + 1;
+  const size_t N = s.in.size() + 1 + s.more_out.size();
   const size_t R = size_t(s.rank);
   if (a.ptrs.size() != N || a.shape.size() != R || a.offsets.size() != N || a.strides.size() != N)
     throw Error(WKF_ERR_INVALID_ARG, "map_pack_args: argument arity does not match the kernel");
@@ -404,7 +439,9 @@ std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a) {
     if (st.size() != R) throw Error(WKF_ERR_INVALID_ARG, "map_pack_args: stride rank mismatch");
     for (uint32_t v : st) put32(b, v);
   }
-  size_t nc = s.prog.consts.empty() ? 1 : s.prog.consts.size();
+  size_t nc = s.prog.consts.size();
+  for (const Program& p : s.more_prog) nc += p.consts.size();
+  nc = std::max<size_t>(1, nc);
   for (size_t i = 0; i < nc; i++) putf(b, i < a.consts.size() ? a.consts[i] : 0.f);
   pad8(b);
   return b;

@@ -48,6 +48,10 @@ struct MapSpec {
   std::vector<MapOperandSpec> in;    // inputs
   MapOperandSpec out;
   Program prog;
+  // Further outputs computed from the same inputs over the same iteration space (one more store each;
+  // shared loads and shared sub-expressions are done once).  Not with tile_dim.
+  std::vector<MapOperandSpec> more_out;
+  std::vector<Program> more_prog;
   MathPolicy math = MathPolicy::Stored;
 };
 constexpr int kMaxRank = 6;
@@ -58,12 +62,12 @@ std::string map_signature(const MapSpec& s);
 std::string map_source(const MapSpec& s);
 // Size in bytes of the argument block and the packer that fills it.
 struct MapArgs {
-  std::vector<void*> ptrs;               // inputs..., out
+  std::vector<void*> ptrs;               // inputs..., out, further outputs...
   uint32_t nwork;                        // number of work items (vectors)
   std::vector<uint32_t> shape;           // coalesced shape; the last entry is in work items
   std::vector<uint32_t> offsets;         // per operand, elements
   std::vector<std::vector<uint32_t>> strides;  // per operand, per dim, elements
-  std::vector<float> consts;
+  std::vector<float> consts;             // of prog, then of every further program
 };
 std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a);
 

@@ -98,10 +98,14 @@ int Resolver::build(ExprBuilder& eb, const NodeP& n, int pairwise_budget) {
   int v;
   // Keep kernels within a sane register / argument budget: past it, a sub-tree is materialised.
   const bool room = eb.prog.ins.size() < 48 && eb.operands.size() < 7;
-  if (eb.split && n.get() == eb.split->cat) {
+  NodeP piece;
+  if (eb.split && !eb.inside_piece && (n->kind == NodeKind::SliceAssign || n->kind == NodeKind::MapLayout))
+    piece = slice_through(n, eb.split->axis, eb.split->start, eb.split->end);
+  if (piece) {
+    // cat([A, B]) (possibly under broadcasts) restricted to this piece's range IS A or B
     const bool was = eb.inside_piece;
     eb.inside_piece = true;  // operands below are already piece-shaped
-    v = build(eb, eb.split->piece, pairwise_budget);
+    v = build(eb, piece, pairwise_budget);
     eb.inside_piece = was;
   } else if (n->kind == NodeKind::ElementWise) {
     int a = build(eb, n->a, pairwise_budget);
@@ -161,6 +165,57 @@ const Node* find_cat2(const Node* n, int depth = 0) {
   return nullptr;
 }
 }  // namespace
+
+// The node that computes `n` restricted to [start, end) along `axis` without computing the rest of `n`,
+// or null when there is no such shortcut: a two-piece cat cut exactly at its seam is one of its pieces,
+// and a broadcast of such a cat is the broadcast of the piece.
+NodeP Resolver::slice_through(const NodeP& n, size_t axis, size_t start, size_t end) {
+  auto key = std::make_tuple(n.get(), axis, start, end);
+  auto it = sliced_.find(key);
+  if (it != sliced_.end()) return it->second;
+  NodeP result;
+  NodeP a, b;
+  size_t cat_axis = 0;
+  if (match_cat2(n.get(), &a, &b, &cat_axis)) {
+    if (cat_axis == axis) {
+      const size_t mid = a->shape[axis];
+      if (start == 0 && end == mid) result = a;
+      else if (start == mid && end == n->shape[axis]) result = b;
+    }
+  } else if (n->kind == NodeKind::MapLayout && n->map_kind == MapKind::Broadcast && axis != n->axis0) {
+    NodeP inner = slice_through(n->a, axis > n->axis0 ? axis - 1 : axis, start, end);
+    if (inner) {
+      auto m = std::make_shared<Node>(*n);
+      m->a = inner;
+      m->shape[axis] = end - start;
+      m->new_shape = m->shape;
+      result = m;
+    }
+  }
+  else if (n->kind == NodeKind::MapLayout && n->map_kind == MapKind::Slice && axis < n->ranges.size() &&
+           n->ranges[axis] == std::make_pair(size_t(0), n->a->shape[axis])) {
+    // a slice that leaves `axis` whole (narrow on another dimension)
+    NodeP inner = slice_through(n->a, axis, start, end);
+    if (inner) {
+      auto m = std::make_shared<Node>(*n);
+      m->a = inner;
+      m->ranges[axis] = std::make_pair(size_t(0), end - start);
+      m->shape[axis] = end - start;
+      result = m;
+    }
+  } else if (n->kind == NodeKind::MapLayout && n->map_kind == MapKind::Transpose) {
+    const size_t inner_axis = axis == n->axis0 ? n->axis1 : axis == n->axis1 ? n->axis0 : axis;
+    NodeP inner = slice_through(n->a, inner_axis, start, end);
+    if (inner) {
+      auto m = std::make_shared<Node>(*n);
+      m->a = inner;
+      m->shape[axis] = end - start;
+      result = m;
+    }
+  }
+  sliced_[key] = result;  // keeps the temporary node alive for the whole resolve (maps are keyed by address)
+  return result;
+}
 
 TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero) {
   TensorData td;
@@ -263,6 +318,7 @@ TensorData Resolver::resolve_root(const NodeP& root) {
   std::set<const Node*>& shared = shared_;
   shared.clear();
   materialized_.clear();
+  sliced_.clear();
   // An element-wise or pair-wise node is inlined into every kernel that uses it,
   // so its second use is also a second use of its inputs: the walk goes through
   // it twice.  Any other node is cut off at its second use.
@@ -282,6 +338,7 @@ TensorData Resolver::resolve_root(const NodeP& root) {
   shared.erase(root.get());
   TensorData out = resolve(root);
   materialized_.clear();
+  sliced_.clear();
   return out;
 }
 
@@ -533,24 +590,43 @@ TensorData Resolver::run_map(const NodeP& root) {
       match_cat2(cat, &pa, &pb, &axis);
       const size_t mid = pa->shape[axis], total = cat->shape[axis];
       TensorData out;
+      CatPiece piece[2];
+      ExprBuilder eb[2];
+      TensorData view[2];
       for (int part = 0; part < 2; part++) {
-        CatPiece piece;
-        piece.cat = cat;
-        piece.piece = part == 0 ? pa : pb;
-        piece.axis = axis;
-        piece.start = part == 0 ? 0 : mid;
-        piece.end = part == 0 ? mid : total;
-        ExprBuilder eb;
-        eb.split = &piece;
-        eb.prog.result = build(eb, root, pairwise_budget_for_map());
-        if (part == 0) out = alloc(root->shape, eb.prog.result_dtype(), false);
+        piece[part].axis = axis;
+        piece[part].start = part == 0 ? 0 : mid;
+        piece[part].end = part == 0 ? mid : total;
+        eb[part].split = &piece[part];
+        eb[part].prog.result = build(eb[part], root, pairwise_budget_for_map());
+        if (part == 0) out = alloc(root->shape, eb[part].prog.result_dtype(), false);
         std::vector<std::pair<size_t, size_t>> r;
         for (size_t d = 0; d < root->shape.size(); d++)
-          r.push_back(d == axis ? std::make_pair(piece.start, piece.end) : std::make_pair(size_t(0), root->shape[d]));
-        TensorData view = out;
-        view.layout = out.layout.slice(r);
-        if (piece.end > piece.start) launch_map(eb.prog, eb.operands, view, false);
+          r.push_back(d == axis ? std::make_pair(piece[part].start, piece[part].end) : std::make_pair(size_t(0), root->shape[d]));
+        view[part] = out;
+        view[part].layout = out.layout.slice(r);
       }
+      if (mid == total - mid && mid > 0) {
+        // Pieces of one shape (rope's two halves): ONE kernel with two stores; the operands the pieces
+        // share (x1, x2, cos, sin) are loaded once.
+        std::vector<TensorData> operands = eb[0].operands;
+        Program second = eb[1].prog;
+        for (Instr& in : second.ins) {
+          if (in.op != Op::Load) continue;
+          const TensorData& td = eb[1].operands[size_t(in.operand)];
+          size_t k = 0;
+          for (; k < operands.size(); k++)
+            if (operands[k].buffer.get() == td.buffer.get() && operands[k].dtype == td.dtype && operands[k].layout == td.layout) break;
+          if (k == operands.size()) operands.push_back(td);
+          in.operand = int(k);
+        }
+        if (operands.size() <= 8) {
+          launch_map(eb[0].prog, operands, view[0], false, {second}, {view[1]});
+          return out;
+        }
+      }
+      for (int part = 0; part < 2; part++)
+        if (piece[part].end > piece[part].start) launch_map(eb[part].prog, eb[part].operands, view[part], false);
       return out;
     }
   }
@@ -574,8 +650,11 @@ TensorData Resolver::run_map(const NodeP& root) {
   return out;
 }
 
-void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place) {
+void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place,
+                          const std::vector<Program>& more_prog, const std::vector<TensorData>& more_out) {
   const std::vector<size_t>& shape = out.layout.shape;
+  for (const TensorData& td : more_out)
+    if (td.layout.shape != shape) invalid("map kernel: outputs of different shapes");
   for (const TensorData& td : in)
     if (td.layout.shape != shape)
       invalid("operand shapes differ: " + dims(td.layout.shape) + " vs " + dims(shape));  // src/pair_wise.rs:92
@@ -598,8 +677,10 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   std::vector<size_t> pshape;
   for (size_t d : order) pshape.push_back(shape[d]);
   std::vector<std::vector<size_t>> strides;
-  for (size_t k = 0; k <= in.size(); k++) {
-    const std::vector<size_t>& st = k < in.size() ? in[k].layout.strides : out.layout.strides;
+  const size_t N = in.size() + 1 + more_out.size();
+  auto td_of = [&](size_t k) -> const TensorData& { return k < in.size() ? in[k] : k == in.size() ? out : more_out[k - in.size() - 1]; };
+  for (size_t k = 0; k < N; k++) {
+    const std::vector<size_t>& st = td_of(k).layout.strides;
     std::vector<size_t> ps;
     for (size_t d : order) ps.push_back(st[d]);
     strides.push_back(ps);
@@ -611,9 +692,6 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   }
   const size_t R = sp.shape.size();
   if (R > size_t(kMaxRank)) throw Error(WKF_ERR_UNSUPPORTED, "map kernel: more than 6 non-mergeable dimensions");
-  const size_t N = in.size() + 1;
-  auto td_of = [&](size_t k) -> const TensorData& { return k < in.size() ? in[k] : out; };
-
   // Vector width: 16 bytes of the widest element type, shrunk until every operand
   // is either unit-stride and aligned or a broadcast along the inner dimension.
   size_t max_elem = 2;
@@ -625,7 +703,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
       size_t inner = sp.strides[k][R - 1];
       if (inner > 1) return false;
       if (inner == 0) {
-        if (k == N - 1) return false;
+        if (k >= in.size()) return false;
         continue;
       }
       if (td_of(k).layout.offset % V) return false;
@@ -642,8 +720,9 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   spec.prog = prog;
   spec.math = st_.exact_math ? MathPolicy::Exact : MathPolicy::Stored;
   // Inputs that run along another dimension than the output (a transposed operand): tiled kernel.
+  spec.more_prog = more_prog;
   if (vec == 1 && R >= 2 && numel >= (size_t(1) << 16) && sp.strides[N - 1][R - 1] == 1 && sp.shape[R - 1] >= 16 &&
-      st_.fusion != FusionMode::Reference) {
+      st_.fusion != FusionMode::Reference && more_out.empty()) {
     int ta = -1;
     for (size_t k = 0; k + 1 < N && ta < 0; k++) {
       if (sp.strides[k][R - 1] <= 1) continue;
@@ -675,7 +754,8 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
     os.inner_stride = vec > 1 ? int(sp.strides[k][R - 1]) : -1;
     if (os.linear) os.inner_stride = vec > 1 ? 1 : -1;
     if (k < in.size()) spec.in.push_back(os);
-    else spec.out = os;
+    else if (k == in.size()) spec.out = os;
+    else spec.more_out.push_back(os);
     bytes += os.linear ? numel * dtype_size(os.dtype) : 0;
   }
   spec.nontemporal = bytes >= st_.nontemporal_bytes;
@@ -695,6 +775,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
     args.strides.push_back(st);
   }
   args.consts = prog.consts;
+  for (const Program& p : more_prog) args.consts.insert(args.consts.end(), p.consts.begin(), p.consts.end());
 
   std::string sig = map_signature(spec);
   wkf_kernel* k = kernel(sig, [&] { return map_source(spec); });
@@ -708,6 +789,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   std::ostringstream d;
   d << "shape=" << dims(sp.shape) << " vec=" << vec << " unroll=" << spec.unroll << " operands=" << N
     << (in_place ? " in_place" : "");
+  if (!more_out.empty()) d << " outputs=" << 1 + more_out.size();
   r.detail = d.str();
   record(std::move(r), k, map_pack_args(spec, args));
 }

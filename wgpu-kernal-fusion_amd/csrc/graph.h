@@ -8,6 +8,7 @@
 #include <map>
 #include <set>
 #include <string>
+#include <tuple>
 #include <vector>
 
 #include "codegen.h"
@@ -52,13 +53,13 @@ class Resolver {
  private:
   TensorData resolve(const NodeP& n);
   TensorData resolve_uncached(const NodeP& n);
-  // When a map kernel consumes cat([A, B], axis), the kernel is run once per piece: the cat
-  // node stands for A (or B) and every other operand is sliced to that piece's range.
+  // When a map kernel consumes cat([A, B], axis), the expression is built once per piece: every cat cut
+  // at that seam (also below broadcasts) stands for its A (or B) and every other operand is sliced to the
+  // piece's range.  Pieces of one shape then share ONE kernel with two stores.
   struct CatPiece {
-    const Node* cat = nullptr;   // the slice_assign node that completes the cat
-    NodeP piece;                 // A or B
     size_t axis = 0, start = 0, end = 0;
   };
+  NodeP slice_through(const NodeP& n, size_t axis, size_t start, size_t end);
   struct ExprBuilder {
     const CatPiece* split = nullptr;
     bool inside_piece = false;
@@ -102,7 +103,9 @@ class Resolver {
   TensorData run_slice_assign(const NodeP& n);
 
   // out[i] = prog(operands[i]) over out.layout.shape; every operand layout has that shape.
-  void launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
+  // `more_prog[j]` (over the same operands) is stored to `more_out[j]` by the same kernel.
+  void launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place,
+                  const std::vector<Program>& more_prog = {}, const std::vector<TensorData>& more_out = {});
   void launch_map_tiled(MapSpec& spec, const Space& sp, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
   TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero);
   TensorData make_contiguous(const TensorData& td);
@@ -114,6 +117,7 @@ class Resolver {
   std::vector<LaunchRecord>* log_;
   std::set<const Node*> shared_;
   std::map<const Node*, TensorData> materialized_;  // nodes with several consumers, computed once per resolve
+  std::map<std::tuple<const Node*, size_t, size_t, size_t>, NodeP> sliced_;  // slice_through results (and owners of its temporary nodes)
 };
 
 }  // namespace wkf
