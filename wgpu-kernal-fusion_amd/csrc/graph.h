@@ -34,6 +34,9 @@ struct Settings {
   int map_unroll = 4;             // work items per thread in large map kernels (WKF_MAP_UNROLL overrides: 1, 2, 4, 8)
   bool exact_math = false;        // every transcendental through an f64 core (MathPolicy::Exact)
   size_t nontemporal_bytes = size_t(32) << 20;  // map kernels moving at least this much use streaming loads/stores
+  int reduce_threads = 0;         // lanes per row in row reduces; 0 = chosen from the shape (WKF_REDUCE_THREADS overrides)
+  int row_threads = 0;            // lanes per row in row kernels; 0 = chosen from the shape (WKF_ROW_THREADS overrides)
+  int reduce_unroll = 0;          // loads in flight per lane in row reduces; 0 = chosen (WKF_REDUCE_UNROLL overrides)
 };
 
 // The iteration space of one kernel seen by all of its operands at once:

@@ -97,6 +97,18 @@ Settings settings_for(wkf_device* dev) {
       if (v == 1 || v == 2 || v == 4 || v == 8) st.map_unroll = v;
     }
     if (const char* nt = getenv("WKF_NONTEMPORAL_BYTES")) st.nontemporal_bytes = size_t(atoll(nt));
+    if (const char* t = getenv("WKF_REDUCE_THREADS")) {
+      int v = atoi(t);
+      if (v >= 1 && v <= 1024 && (v & (v - 1)) == 0) st.reduce_threads = v;
+    }
+    if (const char* t = getenv("WKF_ROW_THREADS")) {
+      int v = atoi(t);
+      if (v >= 1 && v <= 1024 && (v & (v - 1)) == 0) st.row_threads = v;
+    }
+    if (const char* u = getenv("WKF_REDUCE_UNROLL")) {
+      int v = atoi(u);
+      if (v == 1 || v == 2 || v == 4 || v == 8) st.reduce_unroll = v;
+    }
     it = g_settings.emplace(dev, st).first;
   }
   return it->second;
