@@ -131,6 +131,14 @@ int wkf_tensor_arange(wkf_device* dev, int dtype, float start, float end, float 
 /* LazyTensorData::materialize, src/tensor.rs:286-288: run the graph under `t`.
  * The result stays on the device; kernels are timed with a hipEvent pair each. */
 int wkf_tensor_materialize(wkf_tensor* t);
+/* wkf_tensor_materialize / wkf_tensor_as_slice for several tensors of one device in ONE pass over their
+ * joint graph: what they share is computed once, and reductions over the last axis of the same rows (row
+ * max and row sum(exp(x - 1)) of one matrix) run as one kernel that reads the rows once -- the "parallel
+ * reduces" the reference lists as to-do (README.md:20; its resolve, src/compute_graph/mod.rs:241-248,
+ * takes one key per call).  Every launch of the pass is recorded on ts[0] (wkf_tensor_kernel_info).
+ * as_slice_many writes n slices into out[0..n), each to be released with wkf_slice_free. */
+int wkf_tensor_materialize_many(wkf_tensor** ts, int n);
+int wkf_tensor_as_slice_many(wkf_tensor** ts, int n, wkf_slice** out);
 /* Tensor::all_timing_information, src/tensor.rs:556-558: number of kernels the
  * last materialize launched, and for kernel `i` its elapsed time, kind and
  * cache signature. */

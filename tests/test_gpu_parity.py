@@ -286,6 +286,35 @@ def test_long_axis_reductions_of_views(gpu):
     assert np.array_equal(got[5], want[5].to_numpy())
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+def test_tensors_materialised_together(gpu, wkf, dtype):
+    # several roots in one pass: sibling row reductions become one kernel; every value is what the tensor gives alone
+    x = data((300, 1024), -1, 1, dtype, 41)
+    y = data((7, 5, 96), -1, 1, dtype, 42)
+    t, u = wkf.Tensor.new(gpu, x), wkf.Tensor.new(gpu, y)
+    roots = [t.max(1), (t.clone() - 1.0).exp().sum(1) + 2.0, t.min(1), (t * t).sum(1).sqrt(),
+             u.sum(2), u.max(2) * 0.5, u.sum(1), (t * 2.0).exp()]
+    if gpu.is_planner:  # the run that only fills the kernel cache: compile both ways, compute nothing
+        wkf.materialize_many(roots)
+        hip_values_many(roots)
+    together = [s.to_numpy() for s in wkf.as_slice_many(roots)]
+    assert any(k.kind == "row" and "reductions=" in k.detail for k in roots[0].kernels())
+    alone = [r.to_numpy() for r in roots]
+    o, v = OTensor(x), OTensor(y)
+    want = [o.max(1), (o - 1.0).exp().sum(1) + 2.0, o.min(1), (o * o).sum(1).sqrt(), v.sum(2), v.max(2) * 0.5, v.sum(1), (o * 2.0).exp()]
+    rtol = 1e-5 if dtype == np.float32 else 1e-2
+    for i, (g, a, w) in enumerate(zip(together, alone, want)):
+        w = w.to_numpy()
+        assert g.shape == w.shape and g.dtype == w.dtype, i
+        if i in (0, 2, 5):
+            assert np.array_equal(g, w), f"root {i}: max / min are exact"
+        elif i == 7:
+            assert_ulp(g, w, 2, f"root {i}")
+        else:
+            assert np.allclose(g.astype(np.float64), w.astype(np.float64), rtol=rtol, atol=rtol * 50), f"root {i}"
+        assert np.allclose(g.astype(np.float64), a.astype(np.float64), rtol=rtol, atol=rtol * 50), f"root {i} vs alone"
+
+
 def test_reduce_seeds_and_empty_axes(gpu):
     api = HipAPI(gpu)
     ninf = np.full((3, 40), -np.inf, dtype=np.float32)

@@ -269,6 +269,37 @@ def test_few_outputs_over_a_long_axis_fold_in_two_launches(wkf, planner):
         planner.set_fusion(wkf.FUSION_TREE)
 
 
+def test_sibling_row_reductions_share_one_pass(wkf, planner):
+    # README.md:20 of the reference lists "parallel reduces" as to-do; here several tensors are materialised together
+    x = wkf.Tensor.new(planner, np.zeros((512, 2048), dtype=np.float32))
+    a, b, c = x.max(1), (x.clone() - 1.0).exp().sum(1) + 2.0, x.min(1)
+    wkf.materialize_many([a, b, c])
+    ks = a.kernels()
+    assert [k.kind for k in ks] == ["row"] and "reductions=3" in ks[0].detail and "|scalars" in ks[0].signature
+    assert b.kernels() == [] and c.kernels() == []  # the pass is recorded on the first tensor
+    # alone, each is an ordinary reduce
+    assert _kinds(a) == ["red_row"]
+    # a shared producer is computed once for all of its consumers; reductions over other axes run one by one
+    g = x.mat_mul(wkf.Tensor.new(planner, np.zeros((2048, 256), dtype=np.float32)))
+    s0, s1, m = g.sum(0), g.sum(1), g.max(1) * 3.0
+    wkf.materialize_many([s0, s1, m])
+    kinds = [k.kind for k in s0.kernels()]
+    assert kinds.count("gemm") == 1 and kinds.count("row") == 1 and kinds.count("red_col") >= 1 and len(kinds) <= 4
+    # rows too long for the registers of one block: separate (two-launch) reduces
+    y = wkf.Tensor.new(planner, np.zeros((64, 400000), dtype=np.float32))
+    p, q = y.max(1), y.sum(1)
+    wkf.materialize_many([p, q])
+    assert [k.kind for k in p.kernels()] == ["red_row"] * 4
+    planner.set_fusion(wkf.FUSION_REFERENCE)
+    try:
+        wkf.materialize_many([a, c])
+        assert [k.kind for k in a.kernels()] == ["red_row", "red_row"]
+    finally:
+        planner.set_fusion(wkf.FUSION_TREE)
+    with pytest.raises(wkf.WkfError):
+        wkf.materialize_many([])
+
+
 def test_one_binary_serves_every_size_and_constant(wkf, planner):
     before = planner.module_stats()
     t1 = (_x(wkf, planner, (256, 256)) * 3.0) + 5.0

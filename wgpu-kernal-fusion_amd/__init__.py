@@ -46,7 +46,7 @@ EXPORTS = [
     "wkf_tensor_reshape", "wkf_tensor_unsqueeze", "wkf_tensor_slice_assign", "wkf_tensor_cat", "wkf_tensor_silu",
     "wkf_tensor_layer_norm", "wkf_tensor_rope", "wkf_tensor_softmax", "wkf_tensor_softmax_last_dim",
     "wkf_tensor_arange", "wkf_tensor_materialize", "wkf_tensor_kernel_count", "wkf_tensor_kernel_info",
-    "wkf_kernel_source", "wkf_tensor_graphvis", "wkf_tensor_as_slice", "wkf_slice_free", "wkf_slice_rank", "wkf_slice_dtype",
+    "wkf_kernel_source", "wkf_tensor_graphvis", "wkf_tensor_materialize_many", "wkf_tensor_as_slice_many", "wkf_tensor_as_slice", "wkf_slice_free", "wkf_slice_rank", "wkf_slice_dtype",
     "wkf_slice_layout", "wkf_slice_data", "wkf_slice_get",
 ]
 
@@ -120,6 +120,8 @@ def load():
                                            c_char_p, c_size_t]
     lib.wkf_kernel_source.argtypes = [c_char_p, c_char_p, c_size_t, POINTER(c_size_t)]
     lib.wkf_tensor_graphvis.argtypes = [c_void_p, c_char_p, c_size_t, POINTER(c_size_t)]
+    lib.wkf_tensor_materialize_many.argtypes = [POINTER(c_void_p), c_int]
+    lib.wkf_tensor_as_slice_many.argtypes = [POINTER(c_void_p), c_int, POINTER(c_void_p)]
     lib.wkf_tensor_as_slice.argtypes = [c_void_p, POINTER(c_void_p)]
     lib.wkf_slice_free.argtypes = [c_void_p]
     lib.wkf_slice_free.restype = None
@@ -559,6 +561,23 @@ class Tensor:
         """`Tensor::all_timing_information` (src/tensor.rs:556-558): re-materialises, then reports."""
         self.materialize()
         return self.kernels()
+
+
+def materialize_many(tensors):
+    """Materialise several tensors in one pass (shared work once, sibling row reductions in one kernel).
+    The launches are recorded on tensors[0]."""
+    lib = load()
+    arr = (c_void_p * len(tensors))(*[t._h for t in tensors])
+    _check(lib.wkf_tensor_materialize_many(arr, len(tensors)))
+
+
+def as_slice_many(tensors):
+    """`as_slice` for several tensors in one pass over their joint graph; returns one TensorSlice each."""
+    lib = load()
+    arr = (c_void_p * len(tensors))(*[t._h for t in tensors])
+    out = (c_void_p * len(tensors))()
+    _check(lib.wkf_tensor_as_slice_many(arr, len(tensors), out))
+    return [TensorSlice(c_void_p(h)) for h in out]
 
 
 def kernel_source(signature):

@@ -128,7 +128,14 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
         break;
       }
       default: {
-        std::string call = math_call(in.op, h ? "(float)" + a : a, exact_op(p, i, policy), far_variant);
+        const bool exact = exact_op(p, i, policy);
+        if (h && !exact && in.op == Op::Exp) {
+          // f16 result: 2^(x log2 e) on the hardware unit (relative error about 2^-21 for any f16 argument,
+          // a thousand times finer than the f16 grid); the f32 library's exp would cost more than the loads.
+          o << "(_Float16)__builtin_amdgcn_exp2f((float)" << a << " * 0x1.715476p+0f)";
+          break;
+        }
+        std::string call = math_call(in.op, h ? "(float)" + a : a, exact, far_variant);
         o << (h ? "(_Float16)" : "") << call;
       }
     }
@@ -753,7 +760,8 @@ std::string row_signature(const RowSpec& s) {
   for (const auto& i : s.in) o << dtype_name(i.dtype) << 'a' << i.axis_stride << ',';
   o << "|out:" << dtype_name(s.out_dtype);
   for (const auto& st : s.stages) o << "|" << reduce_name(st.rop) << "{" << st.pre.signature() << "}{" << st.post.signature() << "}";
-  o << "|final{" << s.final.signature() << "}";
+  if (s.store_scalars) o << "|scalars";
+  else o << "|final{" << s.final.signature() << "}";
   return o.str();
 }
 
@@ -764,7 +772,9 @@ std::string row_source(const RowSpec& s) {
   const MathPolicy fold_policy = s.exact_math ? MathPolicy::Exact : MathPolicy::Folded;
   // Everything a row kernel stores is combined with a fold result, so it is in the reduction
   // tolerance class (1e-5 relative) as a whole: the f32 library is used throughout.
-  const MathPolicy store_policy = fold_policy;
+  // A stored reduction (no `final`) finishes like any reduce kernel does.
+  const MathPolicy store_policy = s.store_scalars ? (s.exact_math ? MathPolicy::Exact : MathPolicy::Stored) : fold_policy;
+  const int NOUT = s.store_scalars ? int(s.stages.size()) : 1;
   int nc = 0;
   std::vector<int> pre_off, post_off;
   for (const auto& st : s.stages) {
@@ -774,15 +784,15 @@ std::string row_source(const RowSpec& s) {
     nc += int(st.post.consts.size());
   }
   const int final_off = nc;
-  nc += int(s.final.consts.size());
+  if (!s.store_scalars) nc += int(s.final.consts.size());
   std::ostringstream o;
   o << kPrelude;
-  bool math = uses_math(s.final, store_policy);
+  bool math = !s.store_scalars && uses_math(s.final, store_policy);
   for (const auto& st : s.stages) math |= uses_math(st.pre, fold_policy) || uses_math(st.post, store_policy);
   if (math) o << kMath;
   o << kRowHelpers;
-  o << "struct Args { void* p[" << K + 1 << "]; u32 nrows; u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + 1
-    << "]; u32 ostride[" << K + 1 << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
+  o << "struct Args { void* p[" << K + NOUT << "]; u32 nrows; u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
+    << "]; u32 ostride[" << K + NOUT << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
   // operand types as every program sees them: the K full operands, then one scalar per earlier stage
   std::vector<DType> types;
   for (const auto& i : s.in) types.push_back(i.dtype);
@@ -792,7 +802,7 @@ std::string row_source(const RowSpec& s) {
     emit_program(o, s.stages[k].post, "wkf_post" + std::to_string(k), {s.stages[k].pre.result_dtype()}, store_policy);
     types.push_back(s.stages[k].post.result_dtype());
   }
-  emit_program(o, s.final, "wkf_final", types, store_policy);
+  if (!s.store_scalars) emit_program(o, s.final, "wkf_final", types, store_policy);
 
   o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") WKF_ENTRY(const Args a) {\n";
   if (T > 64) o << "  __shared__ float wkf_partial[" << std::max(1, S) << "][" << B / 64 << "];\n";
@@ -858,6 +868,15 @@ std::string row_source(const RowSpec& s) {
     o << "  const " << ctype(st.post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(st.pre.result_dtype()) << ")acc" << k
       << ", a.c + " << post_off[k] << ");\n";
   }
+  if (s.store_scalars) {
+    o << "  if (live && t == 0u) {\n";
+    for (int k = 0; k < S; k++) {
+      const char* st = ctype(s.stages[k].post.result_dtype());
+      o << "    ((" << st << "*)a.p[" << K + k << "])[" << base_expr(K + k) << "] = r" << k << ";\n";
+    }
+    o << "  }\n}\n";
+    return o.str();
+  }
   const char* ot = ctype(s.out_dtype);
   o << "  if (live) {\n";
   o << "    " << ot << "* qo = ((" << ot << "*)a.p[" << K << "]) + (" << base_expr(K) << ");\n";
@@ -877,7 +896,8 @@ std::string row_source(const RowSpec& s) {
 
 std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a) {
   const size_t K = s.in.size(), Ro = size_t(s.outer_rank);
-  if (a.ptrs.size() != K + 1 || a.oshape.size() != Ro || a.offsets.size() != K + 1 || a.ostrides.size() != K + 1)
+  const size_t NP = K + (s.store_scalars ? s.stages.size() : 1);
+  if (a.ptrs.size() != NP || a.oshape.size() != Ro || a.offsets.size() != NP || a.ostrides.size() != NP)
     throw Error(WKF_ERR_INVALID_ARG, "row_pack_args: argument arity does not match the kernel");
   std::vector<unsigned char> b;
   for (void* p : a.ptrs) putp(b, p);
@@ -888,7 +908,7 @@ std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a) {
     if (st.size() != Ro) throw Error(WKF_ERR_INVALID_ARG, "row_pack_args: stride rank mismatch");
     for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? st[d] : 0);
   }
-  size_t nc = s.final.consts.size();
+  size_t nc = s.store_scalars ? 0 : s.final.consts.size();
   for (const auto& st : s.stages) nc += st.pre.consts.size() + st.post.consts.size();
   nc = std::max<size_t>(1, nc);
   for (size_t i = 0; i < nc; i++) putf(b, i < a.consts.size() ? a.consts[i] : 0.f);

@@ -143,16 +143,18 @@ struct RowSpec {
   Program final;                        // same operand numbering as a stage's pre
   DType out_dtype;
   bool exact_math = false;
+  // Parallel reductions: no `final`; output q (one per stage) holds post_q(fold_q) of every row.
+  bool store_scalars = false;
 };
 
 std::string row_signature(const RowSpec& s);
 std::string row_source(const RowSpec& s);
 struct RowArgs {
-  std::vector<void*> ptrs;                        // inputs..., out
+  std::vector<void*> ptrs;                        // inputs..., out (store_scalars: one out per stage)
   uint32_t nrows;
   std::vector<uint32_t> oshape;
-  std::vector<uint32_t> offsets;                  // per operand incl. out
-  std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. out, per outer dim
+  std::vector<uint32_t> offsets;                  // per operand incl. outputs
+  std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. outputs, per outer dim
   std::vector<float> consts;                      // stage 0 pre, stage 0 post, stage 1 pre, ..., final
 };
 std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a);

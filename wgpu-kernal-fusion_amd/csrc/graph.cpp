@@ -342,6 +342,63 @@ TensorData Resolver::resolve_root(const NodeP& root) {
   return out;
 }
 
+// Several roots in one pass: what they share is computed once, and reductions over the last axis of
+// the same rows run as one kernel.  (The reference materialises one tensor per call.)
+std::vector<TensorData> Resolver::resolve_roots(const std::vector<NodeP>& roots) {
+  std::map<const Node*, int> uses;
+  shared_.clear();
+  materialized_.clear();
+  sliced_.clear();
+  std::function<void(const NodeP&)> walk = [&](const NodeP& n) {
+    if (!n) return;
+    const int seen = ++uses[n.get()];
+    if (seen > 2) return;
+    if (seen == 2) {
+      shared_.insert(n.get());
+      if (n->kind != NodeKind::ElementWise && n->kind != NodeKind::PairWise) return;
+    }
+    walk(n->a);
+    walk(n->b);
+  };
+  if (st_.fusion == FusionMode::Tree) {
+    for (const NodeP& r : roots) walk(r);
+    // group the roots that are [a chain above] a reduce over the last axis by the shape they reduce
+    std::map<std::vector<size_t>, std::vector<ReduceRoot>> groups;
+    for (const NodeP& r : roots) {
+      if (materialized_.count(r.get())) continue;
+      ReduceRoot m;
+      m.root = r.get();
+      const Node* cur = r.get();
+      while (cur->kind == NodeKind::ElementWise) {
+        m.chain.push_back(cur);
+        cur = cur->a.get();
+      }
+      if (cur->kind != NodeKind::Reduce || cur->a->shape.empty() || cur->axis != cur->a->shape.size() - 1) continue;
+      bool inner_shared = shared_.count(cur) > 0;
+      for (size_t i = 1; i < m.chain.size(); i++) inner_shared |= shared_.count(m.chain[i]) > 0;
+      if (inner_shared) continue;  // something else needs the reduce's own value
+      m.reduce = cur;
+      bool dup = false;
+      for (const ReduceRoot& o : groups[cur->a->shape]) dup |= o.root == m.root;
+      if (!dup) groups[cur->a->shape].push_back(m);
+    }
+    for (auto& g : groups) {
+      std::vector<TensorData> outs;
+      if (try_parallel_reduces(g.second, &outs))
+        for (size_t i = 0; i < g.second.size(); i++) materialized_[g.second[i].root] = outs[i];
+    }
+  }
+  std::vector<TensorData> out;
+  for (const NodeP& r : roots) {
+    TensorData td = resolve(r);
+    materialized_[r.get()] = td;  // a root listed twice, or used below another root, is computed once
+    out.push_back(td);
+  }
+  materialized_.clear();
+  sliced_.clear();
+  return out;
+}
+
 // ---- row kernels -----------------------------------------------------------------------------
 
 namespace {
@@ -484,19 +541,79 @@ bool Resolver::try_row_kernel(const NodeP& root, TensorData* result) {
   std::map<int, int> loads;
   final.result = row_build(rb, final, memo, loads, root);
   if (!rb.ok || rb.stages.empty() || rb.operands.empty() || rb.operands.size() > 4 || rb.stages.size() > 4) return false;
+  std::vector<TensorData> outs;
+  if (!launch_row(rb, &final, &outs)) return false;
+  *result = outs[0];
+  return true;
+}
+
+// Several reductions over the last axis of the same rows (row max and row sum(exp(x - 1)) of one matrix)
+// in ONE pass: a row kernel whose stages are the reductions and which stores one scalar per stage and row
+// instead of a mapped row.  The reference lists this as to-do (README.md:20) and runs one kernel each.
+bool Resolver::try_parallel_reduces(const std::vector<ReduceRoot>& members, std::vector<TensorData>* outs) {
+  if (st_.fusion != FusionMode::Tree || members.size() < 2 || members.size() > 4) return false;
+  RowBuild rb;
+  rb.shape = members[0].reduce->a->shape;
+  if (rb.shape.empty()) return false;
+  for (const ReduceRoot& m : members) {
+    if (m.reduce->a->shape != rb.shape || m.reduce->axis != rb.shape.size() - 1) return false;
+    RowStage rs;
+    rs.rop = m.reduce->rop;
+    std::map<const Node*, int> pmemo;
+    std::map<int, int> ploads;
+    rs.pre.result = row_build(rb, rs.pre, pmemo, ploads, m.reduce->a);
+    if (!rb.ok) return false;
+    for (const Instr& in : rs.pre.ins)
+      if (in.op == Op::Load && in.operand >= kScalarBase) return false;  // depends on another reduction of the rows
+    Instr ld;
+    ld.op = Op::Load;
+    ld.dtype = rs.pre.result_dtype();
+    ld.operand = 0;
+    rs.post.ins.push_back(ld);
+    int cur = 0;
+    for (size_t i = m.chain.size(); i-- > 0;) {  // the chain above the reduce, innermost first
+      const Node* c = m.chain[i];
+      if (c->op == Op::Sin || c->op == Op::Cos) return false;  // would need the far-argument redo path
+      Instr in;
+      in.op = c->op;
+      in.a = cur;
+      in.dtype = c->dtype;
+      if (is_const_op(c->op)) {
+        in.cslot = int(rs.post.consts.size());
+        rs.post.consts.push_back(c->constant);
+      }
+      rs.post.ins.push_back(in);
+      cur = int(rs.post.ins.size()) - 1;
+    }
+    rs.post.result = cur;
+    rb.stages.push_back(rs);
+  }
+  if (rb.stages.size() != members.size() || rb.operands.empty() || rb.operands.size() > 4) return false;
+  return launch_row(rb, nullptr, outs);
+}
+
+// Plans and launches a row kernel: with `final`, one output of the rows' shape (softmax, RMSNorm);
+// without, one output per stage holding that stage's scalar of every row (parallel reductions).
+bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<TensorData>* outs) {
+  const bool scalars = final_in == nullptr;
+  Program final;
+  if (final_in) final = *final_in;
   const size_t R = rb.shape.size(), axis = R - 1, n = rb.shape[axis];
-  const size_t K = rb.operands.size();
+  const size_t K = rb.operands.size(), S = rb.stages.size();
+  const size_t NOUT = scalars ? S : 1;
 
   RowSpec spec;
-  size_t max_elem = dtype_size(final.result_dtype());
+  size_t max_elem = scalars ? 2 : dtype_size(final.result_dtype());
   for (const TensorData& td : rb.operands) max_elem = std::max(max_elem, dtype_size(td.dtype));
   const int V = int(16 / max_elem);
   if (n == 0 || n % V) return false;
   std::vector<size_t> out_shape(rb.shape.begin(), rb.shape.end() - 1);
-  TensorData out = alloc(rb.shape, final.result_dtype(), false);
   std::vector<std::vector<size_t>> ostr;
   for (const TensorData& td : rb.operands) ostr.push_back(std::vector<size_t>(td.layout.strides.begin(), td.layout.strides.end() - 1));
-  ostr.push_back(std::vector<size_t>(out.layout.strides.begin(), out.layout.strides.end() - 1));
+  // outputs are fresh contiguous tensors: rows of the full shape, or one scalar per row
+  std::vector<size_t> full_strides = Layout::contiguous_strides(rb.shape);
+  for (size_t q = 0; q < NOUT; q++)
+    ostr.push_back(scalars ? Layout::contiguous_strides(out_shape) : std::vector<size_t>(full_strides.begin(), full_strides.end() - 1));
   Space sp = coalesce(out_shape, ostr);
   const size_t Ro = sp.shape.size();
   if (Ro > 3) return false;
@@ -525,10 +642,6 @@ bool Resolver::try_row_kernel(const NodeP& root, TensorData* result) {
   if (NV > 16 || NV * V * K > 128) return false;
   size_t nrows = 1;
   for (size_t d : out_shape) nrows *= d;
-  if (nrows == 0) {
-    *result = out;
-    return true;
-  }
   if (nrows > 0xffffffffull) return false;
 
   // operand numbering: full operands 0..K-1, then the scalars
@@ -545,14 +658,20 @@ bool Resolver::try_row_kernel(const NodeP& root, TensorData* result) {
   spec.vectors_per_lane = int(NV);
   spec.stages = rb.stages;
   spec.final = final;
-  spec.out_dtype = final.result_dtype();
+  spec.store_scalars = scalars;
+  spec.out_dtype = scalars ? DType::F32 : final.result_dtype();
   spec.exact_math = st_.exact_math;
+
+  outs->clear();
+  for (size_t q = 0; q < NOUT; q++)
+    outs->push_back(scalars ? alloc(out_shape, rb.stages[q].post.result_dtype(), false) : alloc(rb.shape, final.result_dtype(), false));
+  if (nrows == 0) return true;
 
   RowArgs args;
   args.nrows = uint32_t(nrows);
   for (size_t d = 0; d < Ro; d++) args.oshape.push_back(to_u32(sp.shape[d], "shape"));
-  for (size_t k = 0; k <= K; k++) {
-    const TensorData& td = k < K ? rb.operands[k] : out;
+  for (size_t k = 0; k < K + NOUT; k++) {
+    const TensorData& td = k < K ? rb.operands[k] : (*outs)[k - K];
     args.ptrs.push_back(element_ptr(td));
     args.offsets.push_back(to_u32(td.layout.offset, "offset"));
     std::vector<uint32_t> st;
@@ -575,10 +694,10 @@ bool Resolver::try_row_kernel(const NodeP& root, TensorData* result) {
   r.block[0] = uint32_t(spec.block);
   std::ostringstream d;
   d << "rows=" << nrows << " n=" << n << " vec=" << V << " threads_per_row=" << T << " vectors_per_lane=" << NV << " stages="
-    << rb.stages.size() << " operands=" << K + 1;
+    << rb.stages.size() << " operands=" << K + NOUT;
+  if (scalars) d << " reductions=" << S;
   r.detail = d.str();
   record(std::move(r), k, row_pack_args(spec, args));
-  *result = out;
   return true;
 }
 

@@ -52,6 +52,8 @@ class Resolver {
   Resolver(wkf_device* dev, const Settings& st, std::vector<LaunchRecord>* log) : dev_(dev), st_(st), log_(log) {}
   // Entry point: materialise `root` (ComputeGraph::resolve, src/compute_graph/mod.rs:241-248).
   TensorData resolve_root(const NodeP& root);
+  // Several tensors in one pass (shared sub-graphs once, sibling row reductions in one kernel).
+  std::vector<TensorData> resolve_roots(const std::vector<NodeP>& roots);
 
  private:
   TensorData resolve(const NodeP& n);
@@ -84,6 +86,13 @@ class Resolver {
   // or the layouts do not fit; the caller then takes the ordinary path.
   struct RowBuild;
   bool try_row_kernel(const NodeP& root, TensorData* out);
+  struct ReduceRoot {
+    const Node* root = nullptr;         // [chain above] reduce
+    const Node* reduce = nullptr;
+    std::vector<const Node*> chain;     // element-wise nodes above the reduce, outermost first
+  };
+  bool try_parallel_reduces(const std::vector<ReduceRoot>& members, std::vector<TensorData>* outs);
+  bool launch_row(RowBuild& rb, const Program* final, std::vector<TensorData>* outs);
   int row_build(RowBuild& rb, Program& prog, std::map<const Node*, int>& memo, std::map<int, int>& loads, const NodeP& n);
   TensorData run_reduce(const NodeP& reduce, const std::vector<const Node*>& post_chain);
   // One reduce launch: fold `pre(operands)` over `axis`, then (unless `raw`) round to `fold_dtype` and apply `post`.

@@ -723,6 +723,27 @@ int wkf_tensor_materialize(wkf_tensor* t) {
   });
 }
 
+static std::vector<TensorData> materialize_many(wkf_tensor** ts, int n, const char* who) {
+  need(ts, who);
+  if (n <= 0) invalid(std::string(who) + ": no tensors");
+  std::vector<NodeP> roots;
+  for (int i = 0; i < n; i++) {
+    need(ts[i], who);
+    if (ts[i]->dev != ts[0]->dev) invalid(std::string(who) + ": tensors of different devices");
+    for (LaunchRecord& r : ts[i]->launches)
+      if (r.timer) wkf_timer_destroy(r.timer);
+    ts[i]->launches.clear();
+    roots.push_back(ts[i]->node);
+  }
+  // every launch of the joint pass is recorded on the first tensor
+  Resolver res(ts[0]->dev, settings_for(ts[0]->dev), &ts[0]->launches);
+  return res.resolve_roots(roots);
+}
+
+int wkf_tensor_materialize_many(wkf_tensor** ts, int n) {
+  return guarded([&] { materialize_many(ts, n, "wkf_tensor_materialize_many"); });
+}
+
 int wkf_tensor_kernel_count(const wkf_tensor* t) { return t ? int(t->launches.size()) : -1; }
 
 static void copy_str(const std::string& s, char* out, size_t cap) {
@@ -805,6 +826,24 @@ std::string graph_dot(const NodeP& root) {
 }
 }  // namespace
 }  // extern "C++"
+
+int wkf_tensor_as_slice_many(wkf_tensor** ts, int n, wkf_slice** out) {
+  return guarded([&] {
+    need(out, "wkf_tensor_as_slice_many");
+    std::vector<TensorData> tds = materialize_many(ts, n, "wkf_tensor_as_slice_many");
+    std::vector<std::unique_ptr<wkf_slice>> slices;
+    for (const TensorData& td : tds) {
+      std::unique_ptr<wkf_slice> s(new wkf_slice());
+      s->layout = td.layout;
+      s->dtype = td.dtype;
+      s->bytes.resize(wkf_buffer_size(td.buffer.get()));
+      int rc = wkf_buffer_download(td.buffer.get(), 0, s->bytes.data(), s->bytes.size());
+      if (rc != WKF_OK) throw Error(rc, wkf_last_error());
+      slices.push_back(std::move(s));
+    }
+    for (int i = 0; i < n; i++) out[i] = slices[size_t(i)].release();
+  });
+}
 
 int wkf_tensor_graphvis(const wkf_tensor* t, char* out, size_t cap, size_t* needed) {
   return guarded([&] {
