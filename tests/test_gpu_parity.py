@@ -507,7 +507,10 @@ def gemm_check(got, a, b, tol):
 
 
 GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100, 200, 50), (255, 257, 63),
-               (256, 256, 64), (256, 256, 32), (512, 256, 128), (256, 512, 320), (768, 512, 96), (256, 256, 1000)]
+               (256, 256, 64), (256, 256, 32), (512, 256, 128), (256, 512, 320), (768, 512, 96), (256, 256, 1000),
+               # ragged shapes on the MFMA kernels (edge tiles): rows 16-byte aligned, nothing a multiple of the tile
+               (100, 200, 56), (300, 264, 72), (257, 520, 1000), (1000, 40, 328), (16, 1024, 24), (700, 8, 512),
+               (513, 776, 200)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

@@ -300,6 +300,25 @@ def test_sibling_row_reductions_share_one_pass(wkf, planner):
         wkf.materialize_many([])
 
 
+def test_mat_mul_kernel_choice(wkf, planner):
+    def detail(m, n, k, dtype):
+        t = _x(wkf, planner, (m, k), dtype).mat_mul(_x(wkf, planner, (k, n), dtype, seed=1))
+        assert _kinds(t) == ["gemm"]
+        return t.kernels()[0].detail
+
+    assert detail(512, 256, 128, np.float16).endswith("mfma 256x256 tiles")
+    assert detail(512, 256, 96, np.float32).endswith("mfma 256x256 tiles")
+    # not a multiple of the tile but every row 16-byte aligned: the same MFMA kernel with edge handling
+    assert detail(300, 264, 72, np.float16).endswith("mfma 256x256 tiles edge")
+    assert detail(300, 260, 68, np.float32).endswith("mfma 256x256 tiles edge")
+    # unaligned rows or tiny problems: the generic kernel
+    assert detail(300, 262, 72, np.float16).endswith("generic")
+    assert detail(3, 7, 5, np.float32).endswith("generic")
+    # a transposed operand is copied into a dense buffer first (tiled copy), then multiplied
+    t = _x(wkf, planner, (256, 512), np.float16).transpose(0, 1).mat_mul(_x(wkf, planner, (256, 256), np.float16, seed=1))
+    assert _kinds(t) == ["map", "gemm"] and "tiled" in t.kernels()[0].detail
+
+
 def test_one_binary_serves_every_size_and_constant(wkf, planner):
     before = planner.module_stats()
     t1 = (_x(wkf, planner, (256, 256)) * 3.0) + 5.0

@@ -163,7 +163,9 @@ std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a);
 // K4 of the reference (src/matmul.rs:56-155) re-designed for MFMA: hand-written
 // kernels (kernels/gemm_*.hip.inc), chosen by dtype and by whether the shape is
 // a multiple of the 256 x 256 x BK tile.
-enum class GemmKind { MfmaF16, MfmaF32, Generic };
+// The *Edge kinds are the same kernels compiled with edge handling for shapes that are not multiples of
+// the tile (rows of A and B still have to start 16-byte aligned).
+enum class GemmKind { MfmaF16, MfmaF32, MfmaF16Edge, MfmaF32Edge, Generic };
 GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k);
 std::string gemm_signature(GemmKind kind, DType dt);
 std::string gemm_source(GemmKind kind, DType dt);

@@ -19,9 +19,15 @@ const char* const kGemmGeneric =
 }  // namespace
 
 GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k) {
-  if (m == 0 || n == 0 || k == 0 || m % 256 || n % 256) return GemmKind::Generic;
-  if (dt == DType::F16 && k % 64 == 0) return GemmKind::MfmaF16;
-  if (dt == DType::F32 && k % 32 == 0) return GemmKind::MfmaF32;
+  if (m == 0 || n == 0 || k == 0) return GemmKind::Generic;
+  const bool whole = m % 256 == 0 && n % 256 == 0;
+  if (dt == DType::F16 && whole && k % 64 == 0) return GemmKind::MfmaF16;
+  if (dt == DType::F32 && whole && k % 32 == 0) return GemmKind::MfmaF32;
+  // ragged shapes keep the MFMA kernels as long as every row of A and B starts on a 16-byte boundary
+  // and the problem is worth a 256 x 256 tile; tiny or unaligned ones take the generic kernel
+  const size_t chunk = dt == DType::F16 ? 8 : 4;
+  if (k % chunk == 0 && n % chunk == 0 && m >= 16 && n >= 16 && m * n * k >= (size_t(1) << 18))
+    return dt == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
   return GemmKind::Generic;
 }
 
@@ -29,6 +35,8 @@ std::string gemm_signature(GemmKind kind, DType dt) {
   switch (kind) {
     case GemmKind::MfmaF16: return "gemm|gfx950|f16|mfma32x32x16|256x256x64|w2x2";
     case GemmKind::MfmaF32: return "gemm|gfx950|f32|mfma32x32x2|256x256x32|w2x2";
+    case GemmKind::MfmaF16Edge: return "gemm|gfx950|f16|mfma32x32x16|256x256x64|w2x2|edge";
+    case GemmKind::MfmaF32Edge: return "gemm|gfx950|f32|mfma32x32x2|256x256x32|w2x2|edge";
     case GemmKind::Generic: return std::string("gemm|gfx950|") + dtype_name(dt) + "|generic|64x64x16";
   }
   return "";
@@ -38,6 +46,8 @@ std::string gemm_source(GemmKind kind, DType dt) {
   switch (kind) {
     case GemmKind::MfmaF16: return kGemmF16;
     case GemmKind::MfmaF32: return kGemmF32;
+    case GemmKind::MfmaF16Edge: return std::string("#define WKF_EDGE 1\n") + kGemmF16;
+    case GemmKind::MfmaF32Edge: return std::string("#define WKF_EDGE 1\n") + kGemmF32;
     case GemmKind::Generic:
       return std::string("#define WKF_T ") + (dt == DType::F32 ? "float" : "_Float16") + "\n" + kGemmGeneric;
   }
@@ -83,10 +93,13 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.grid[1] = uint32_t((M + 63) / 64);
     if (r.grid[1] > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many rows for the generic kernel");
   } else {
-    r.grid[0] = uint32_t((M / 256) * (N / 256));
+    const size_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    if (tiles > 0x7fffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
+    r.grid[0] = uint32_t(tiles);
   }
   std::ostringstream d;
   d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : " mfma 256x256 tiles");
+  if (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge) d << " edge";
   r.detail = d.str();
   record(std::move(r), k, bytes);
   return out;
