@@ -510,7 +510,11 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                (256, 256, 64), (256, 256, 32), (512, 256, 128), (256, 512, 320), (768, 512, 96), (256, 256, 1000),
                # ragged shapes on the MFMA kernels (edge tiles): rows 16-byte aligned, nothing a multiple of the tile
                (100, 200, 56), (300, 264, 72), (257, 520, 1000), (1000, 40, 328), (16, 1024, 24), (700, 8, 512),
-               (513, 776, 200)]
+               (513, 776, 200),
+               # a handful of rows (decode): the bandwidth kernel, K cut into slices, then a reduce over the slices
+               # few tiles over a long K: K is cut into slices across the grid (f32 partial sums + a reduce)
+               (300, 264, 2048), (128, 1032, 4096), (512, 512, 8192), (256, 256, 2048), (40, 512, 1096),
+               (1, 1024, 512), (5, 2048, 300), (16, 520, 1000), (8, 264, 4096), (2, 96, 8192), (3, 4104, 77)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

@@ -1,4 +1,5 @@
 // mat_mul: UntypedMatMul::run_with_query of the reference (src/matmul.rs:157-205).
+#include <algorithm>
 #include <cstring>
 #include <sstream>
 
@@ -16,6 +17,10 @@ const char* const kGemmF32 =
 const char* const kGemmGeneric =
 #include "kernels/gemm_generic.hip.inc"
     ;
+const char* const kGemmSkinny =
+#include "kernels/gemm_skinny.hip.inc"
+    ;
+constexpr size_t kSkinnyRows = 16;  // most rows of A the bandwidth kernel takes (accumulators: rows x 8 per lane)
 }  // namespace
 
 GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k) {
@@ -66,21 +71,109 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // right for contiguous operands; a view is copied into a dense buffer first.
   a = make_contiguous(a);
   b = make_contiguous(b);
-  TensorData out = alloc({M, N}, a.dtype, false);
-  if (M == 0 || N == 0) return out;
+  if (M == 0 || N == 0) return alloc({M, N}, a.dtype, false);
   if (M > 0xffffffffull || N > 0xffffffffull || K > 0xffffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: dimension does not fit 32 bits");
 
+  // A handful of rows (decode): reading B once is all the work -> the bandwidth kernel, K cut into slices
+  // across the grid, then one reduce launch that adds the slices and rounds to the tensor dtype.
+  const size_t V = a.dtype == DType::F16 ? 8 : 4;
+  if (st_.fusion == FusionMode::Tree && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
+    const size_t esize = dtype_size(a.dtype);
+    const size_t colblocks = (N + 256 * V - 1) / (256 * V);
+    size_t S = (1024 + colblocks - 1) / colblocks;
+    S = std::min(S, std::max<size_t>(1, K * esize / (8 * M)));  // partial sums stay under half of B's bytes
+    S = std::min(S, K / 16);
+    S = std::max<size_t>(S, 1);
+    size_t chunk = (K + S - 1) / S;
+    chunk = (chunk + 3) & ~size_t(3);
+    S = (K + chunk - 1) / chunk;
+    if (S > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many K slices");
+    TensorData part = alloc({S, M, N}, DType::F32, false);
+    std::ostringstream sg;
+    sg << "gemm|gfx950|" << dtype_name(a.dtype) << "|skinny|m" << M << "|v" << V;
+    const std::string sig = sg.str();
+    wkf_kernel* k = kernel(sig, [&] {
+      std::ostringstream src;
+      src << "#define WKF_T " << (a.dtype == DType::F32 ? "float" : "_Float16") << "\n#define WKF_V " << V << "\n#define WKF_M " << M
+          << "\n" << kGemmSkinny;
+      return src.str();
+    });
+    struct {
+      const void* a;
+      const void* b;
+      void* part;
+      uint32_t m, n, k, chunk;
+    } sargs = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(part.buffer.get()),
+               uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(chunk)};
+    std::vector<unsigned char> sbytes(sizeof(sargs));
+    memcpy(sbytes.data(), &sargs, sizeof(sargs));
+    LaunchRecord r;
+    r.kind = "gemm";
+    r.signature = sig;
+    r.block[0] = 256;
+    r.grid[0] = uint32_t(colblocks);
+    r.grid[1] = uint32_t(S);
+    std::ostringstream d;
+    d << "m=" << M << " n=" << N << " k=" << K << " skinny slices=" << S;
+    r.detail = d.str();
+    record(std::move(r), k, sbytes);
+
+    ReduceJob fold;
+    Instr ld;
+    ld.op = Op::Load;
+    ld.dtype = DType::F32;
+    ld.operand = 0;
+    fold.pre.ins.push_back(ld);
+    fold.pre.result = 0;
+    ld.dtype = a.dtype;
+    fold.post.ins.push_back(ld);
+    fold.post.result = 0;
+    fold.operands = {part};
+    fold.axis = 0;
+    fold.rop = ReduceOp::Sum;
+    fold.fold_dtype = a.dtype;
+    return launch_reduce(fold);
+  }
+
   const GemmKind kind = gemm_pick(a.dtype, M, N, K);
+  const bool mfma = kind != GemmKind::Generic;
+  // A few tiles over a long K leave most compute units idle: cut K into slices across blockIdx.y
+  // (f32 partial sums per slice, then one reduce launch), as long as the partial sums stay below
+  // the bytes of A and B.
+  size_t slices = 1, kchunk = 0;
+  if (mfma && st_.fusion == FusionMode::Tree) {
+    wkf_props props;
+    if (wkf_device_props(dev_, &props) != WKF_OK) throw Error(WKF_ERR_HIP, wkf_last_error());
+    const size_t cus = size_t(std::max(1, props.compute_units));
+    const size_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
+    const size_t bk = a.dtype == DType::F16 ? 64 : 32;
+    if (tiles * 2 <= cus && K >= 1024) {
+      size_t S = std::min((cus + tiles - 1) / tiles, K / 512);
+      while (S > 1 && S * M * N * 4 > (M * K + K * N) * dtype_size(a.dtype)) S--;
+      if (S > 1) {
+        kchunk = (K + S - 1) / S;
+        kchunk = (kchunk + bk - 1) / bk * bk;
+        slices = (K + kchunk - 1) / kchunk;
+      }
+    }
+  }
+  const bool split = slices > 1;
+  TensorData out = split ? alloc({slices, M, N}, DType::F32, false) : alloc({M, N}, a.dtype, false);
   std::string sig = gemm_signature(kind, a.dtype);
-  wkf_kernel* k = kernel(sig, [&] { return gemm_source(kind, a.dtype); });
+  if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
+  wkf_kernel* k = kernel(sig, [&] {
+    if (!split) return gemm_source(kind, a.dtype);
+    const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
+    return std::string("#define WKF_SPLITK 1\n") + gemm_source(base, a.dtype);
+  });
 
   struct {
     const void* a;
     const void* b;
     void* c;
-    uint32_t m, n, k, pad;
+    uint32_t m, n, k, kchunk;
   } args = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(out.buffer.get()),
-            uint32_t(M), uint32_t(N), uint32_t(K), 0};
+            uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(kchunk)};
   std::vector<unsigned char> bytes(sizeof(args));
   memcpy(bytes.data(), &args, sizeof(args));
 
@@ -96,12 +189,31 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     const size_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
     if (tiles > 0x7fffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
     r.grid[0] = uint32_t(tiles);
+    r.grid[1] = uint32_t(slices);
   }
   std::ostringstream d;
   d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : " mfma 256x256 tiles");
   if (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge) d << " edge";
+  if (split) d << " slices=" << slices;
   r.detail = d.str();
   record(std::move(r), k, bytes);
+  if (split) {
+    ReduceJob fold;
+    Instr ld;
+    ld.op = Op::Load;
+    ld.dtype = DType::F32;
+    ld.operand = 0;
+    fold.pre.ins.push_back(ld);
+    fold.pre.result = 0;
+    ld.dtype = a.dtype;
+    fold.post.ins.push_back(ld);
+    fold.post.result = 0;
+    fold.operands = {out};
+    fold.axis = 0;
+    fold.rop = ReduceOp::Sum;
+    fold.fold_dtype = a.dtype;
+    return launch_reduce(fold);
+  }
   return out;
 }
 
