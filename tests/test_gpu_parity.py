@@ -529,6 +529,24 @@ def test_mat_mul(gpu, m, n, k, dtype, tol):
     gemm_check(got, a, b, tol)
 
 
+BT_SHAPES = [(256, 512, 128), (300, 264, 2048), (100, 136, 72), (513, 260, 328), (1, 1024, 512), (7, 520, 1000),
+             (32, 264, 4096), (2, 4100, 96), (20, 100, 64), (3, 5, 7), (33, 2048, 1024)]
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
+@pytest.mark.parametrize("m,n,k", BT_SHAPES, ids=[f"{m}x{n}x{k}" for m, n, k in BT_SHAPES])
+def test_mat_mul_with_a_transposed_weight(gpu, m, n, k, dtype, tol):
+    # x * W^T with W [N, K] dense (the linear-layer form): read as it lies by the MFMA kernels, streamed once at
+    # decode sizes (M <= 32), copied first only when its rows are unaligned or the problem is tiny
+    rng = np.random.default_rng(m * 7919 + n * 104729 + k)
+    a = rng.standard_normal((m, k)).astype(dtype)
+    w = rng.standard_normal((n, k)).astype(dtype)
+    api = HipAPI(gpu)
+    got = hip_values(api.tensor(a).mat_mul(api.tensor(w).transpose(0, 1)))
+    assert got.dtype == dtype
+    gemm_check(got, a, np.ascontiguousarray(w.T), tol)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
 def test_mat_mul_identities_and_views(gpu, dtype):
     rng = np.random.default_rng(23)

@@ -318,9 +318,21 @@ def test_mat_mul_kernel_choice(wkf, planner):
     s = _x(wkf, planner, (4, 4096), np.float16).mat_mul(_x(wkf, planner, (4096, 2048), np.float16, seed=1))
     assert _kinds(s) == ["gemm", "red_col"] and "skinny" in s.kernels()[0].detail and s.shape() == (4, 2048)
     assert s.datatype() == wkf.F16 and "fold:f16" in s.kernels()[1].signature
-    # a transposed operand is copied into a dense buffer first (tiled copy), then multiplied
+    # a transposed A is copied into a dense buffer first (tiled copy), then multiplied
     t = _x(wkf, planner, (256, 512), np.float16).transpose(0, 1).mat_mul(_x(wkf, planner, (256, 256), np.float16, seed=1))
     assert _kinds(t) == ["map", "gemm"] and "tiled" in t.kernels()[0].detail
+    # x * W^T for a dense W [N, K] needs no copy: the MFMA kernels read W as it lies ...
+    w = _x(wkf, planner, (512, 256), np.float16, seed=2)
+    t = _x(wkf, planner, (256, 256), np.float16).mat_mul(w.transpose(0, 1))
+    assert _kinds(t) == ["gemm"] and t.kernels()[0].detail.endswith("B^T") and "|bt" in t.kernels()[0].signature
+    # ... and with a handful of rows W is streamed once through MFMA operands (decode)
+    t = _x(wkf, planner, (2, 256), np.float16).mat_mul(w.transpose(0, 1))
+    assert _kinds(t)[0] == "gemm" and "skinny B^T" in t.kernels()[0].detail and t.shape() == (2, 512)
+    planner.set_fusion(wkf.FUSION_REFERENCE)
+    try:
+        assert _kinds(_x(wkf, planner, (256, 256), np.float16).mat_mul(w.transpose(0, 1))) == ["map", "gemm"]
+    finally:
+        planner.set_fusion(wkf.FUSION_TREE)
 
 
 def test_one_binary_serves_every_size_and_constant(wkf, planner):

@@ -166,7 +166,7 @@ std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a);
 // The *Edge kinds are the same kernels compiled with edge handling for shapes that are not multiples of
 // the tile (rows of A and B still have to start 16-byte aligned).
 enum class GemmKind { MfmaF16, MfmaF32, MfmaF16Edge, MfmaF32Edge, Generic };
-GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k);
+GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k, bool b_transposed = false);
 std::string gemm_signature(GemmKind kind, DType dt);
 std::string gemm_source(GemmKind kind, DType dt);
 

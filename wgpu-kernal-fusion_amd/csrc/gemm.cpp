@@ -20,10 +20,13 @@ const char* const kGemmGeneric =
 const char* const kGemmSkinny =
 #include "kernels/gemm_skinny.hip.inc"
     ;
+const char* const kGemmSkinnyBt =
+#include "kernels/gemm_skinny_bt.hip.inc"
+    ;
 constexpr size_t kSkinnyRows = 16;  // most rows of A the bandwidth kernel takes (accumulators: rows x 8 per lane)
 }  // namespace
 
-GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k) {
+GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k, bool b_transposed) {
   if (m == 0 || n == 0 || k == 0) return GemmKind::Generic;
   const bool whole = m % 256 == 0 && n % 256 == 0;
   if (dt == DType::F16 && whole && k % 64 == 0) return GemmKind::MfmaF16;
@@ -31,7 +34,7 @@ GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k) {
   // ragged shapes keep the MFMA kernels as long as every row of A and B starts on a 16-byte boundary
   // and the problem is worth a 256 x 256 tile; tiny or unaligned ones take the generic kernel
   const size_t chunk = dt == DType::F16 ? 8 : 4;
-  if (k % chunk == 0 && n % chunk == 0 && m >= 16 && n >= 16 && m * n * k >= (size_t(1) << 18))
+  if (k % chunk == 0 && (b_transposed || n % chunk == 0) && m >= 16 && n >= 16 && m * n * k >= (size_t(1) << 18))
     return dt == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
   return GemmKind::Generic;
 }
@@ -70,14 +73,78 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // The reference kernel ignores strides and offsets (src/matmul.rs:96-103), which is only
   // right for contiguous operands; a view is copied into a dense buffer first.
   a = make_contiguous(a);
-  b = make_contiguous(b);
+  // ... except B = transpose(W) of a dense W[N][K] (x * W^T, the linear-layer form): the MFMA kernels read
+  // it as it lies (k contiguous), when its rows are 16-byte aligned and the problem is worth a tile.
+  const bool b_is_t = st_.fusion == FusionMode::Tree && b.layout.offset == 0 && K > 1 && N > 1 && b.layout.strides[0] == 1 &&
+                      b.layout.strides[1] == K;
+  const size_t V = a.dtype == DType::F16 ? 8 : 4;
+  // ... and with up to 32 rows of A (decode) W is streamed once, straight into MFMA operands
+  const bool skinny_bt = b_is_t && M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);
+  bool bt = false;
+  if (skinny_bt) {
+    // handled below
+  } else if (b_is_t && gemm_pick(a.dtype, M, N, K, true) != GemmKind::Generic) {
+    bt = true;
+  } else {
+    b = make_contiguous(b);
+  }
   if (M == 0 || N == 0) return alloc({M, N}, a.dtype, false);
   if (M > 0xffffffffull || N > 0xffffffffull || K > 0xffffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: dimension does not fit 32 bits");
-
+  auto fold_slices = [&](const TensorData& part) {
+    // adds the f32 partial sums of the K slices ([S][M][N]) and rounds to the tensor dtype
+    ReduceJob fold;
+    Instr ld;
+    ld.op = Op::Load;
+    ld.dtype = DType::F32;
+    ld.operand = 0;
+    fold.pre.ins.push_back(ld);
+    fold.pre.result = 0;
+    ld.dtype = a.dtype;
+    fold.post.ins.push_back(ld);
+    fold.post.result = 0;
+    fold.operands = {part};
+    fold.axis = 0;
+    fold.rop = ReduceOp::Sum;
+    fold.fold_dtype = a.dtype;
+    return launch_reduce(fold);
+  };
+  if (skinny_bt) {
+    const size_t kblock = 128 / dtype_size(a.dtype);  // 128 bytes of every row per step
+    const size_t gridx = (N + 127) / 128;
+    size_t S = (2048 + gridx - 1) / gridx;
+    S = std::min(S, std::max<size_t>(1, K * dtype_size(a.dtype) / (8 * M)));  // partial sums stay under half of W's bytes
+    S = std::min(S, std::max<size_t>(1, K / (2 * kblock)));
+    size_t chunk = (K + S - 1) / S;
+    chunk = (chunk + kblock - 1) / kblock * kblock;
+    S = (K + chunk - 1) / chunk;
+    if (S > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many K slices");
+    TensorData part = alloc({S, M, N}, DType::F32, false);
+    const std::string sig = std::string("gemm|gfx950|") + dtype_name(a.dtype) + "|skinny_bt|mfma32x32";
+    wkf_kernel* k = kernel(sig, [&] { return std::string("#define WKF_H ") + (a.dtype == DType::F16 ? "1" : "0") + "\n" + kGemmSkinnyBt; });
+    struct {
+      const void* a;
+      const void* w;
+      void* part;
+      uint32_t m, n, k, chunk;
+    } sargs = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(part.buffer.get()),
+               uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(chunk)};
+    std::vector<unsigned char> sbytes(sizeof(sargs));
+    memcpy(sbytes.data(), &sargs, sizeof(sargs));
+    LaunchRecord r;
+    r.kind = "gemm";
+    r.signature = sig;
+    r.block[0] = 256;
+    r.grid[0] = uint32_t(gridx);
+    r.grid[1] = uint32_t(S);
+    std::ostringstream d;
+    d << "m=" << M << " n=" << N << " k=" << K << " skinny B^T slices=" << S;
+    r.detail = d.str();
+    record(std::move(r), k, sbytes);
+    return fold_slices(part);
+  }
   // A handful of rows (decode): reading B once is all the work -> the bandwidth kernel, K cut into slices
   // across the grid, then one reduce launch that adds the slices and rounds to the tensor dtype.
-  const size_t V = a.dtype == DType::F16 ? 8 : 4;
-  if (st_.fusion == FusionMode::Tree && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
+  if (st_.fusion == FusionMode::Tree && !bt && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
     const size_t esize = dtype_size(a.dtype);
     const size_t colblocks = (N + 256 * V - 1) / (256 * V);
     size_t S = (1024 + colblocks - 1) / colblocks;
@@ -118,24 +185,10 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.detail = d.str();
     record(std::move(r), k, sbytes);
 
-    ReduceJob fold;
-    Instr ld;
-    ld.op = Op::Load;
-    ld.dtype = DType::F32;
-    ld.operand = 0;
-    fold.pre.ins.push_back(ld);
-    fold.pre.result = 0;
-    ld.dtype = a.dtype;
-    fold.post.ins.push_back(ld);
-    fold.post.result = 0;
-    fold.operands = {part};
-    fold.axis = 0;
-    fold.rop = ReduceOp::Sum;
-    fold.fold_dtype = a.dtype;
-    return launch_reduce(fold);
+    return fold_slices(part);
   }
 
-  const GemmKind kind = gemm_pick(a.dtype, M, N, K);
+  const GemmKind kind = gemm_pick(a.dtype, M, N, K, bt);
   const bool mfma = kind != GemmKind::Generic;
   // A few tiles over a long K leave most compute units idle: cut K into slices across blockIdx.y
   // (f32 partial sums per slice, then one reduce launch), as long as the partial sums stay below
@@ -161,10 +214,12 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   TensorData out = split ? alloc({slices, M, N}, DType::F32, false) : alloc({M, N}, a.dtype, false);
   std::string sig = gemm_signature(kind, a.dtype);
   if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
+  if (bt) sig += "|bt";
   wkf_kernel* k = kernel(sig, [&] {
-    if (!split) return gemm_source(kind, a.dtype);
+    std::string src = bt ? "#define WKF_BT 1\n" : "";
+    if (!split) return src + gemm_source(kind, a.dtype);
     const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
-    return std::string("#define WKF_SPLITK 1\n") + gemm_source(base, a.dtype);
+    return src + "#define WKF_SPLITK 1\n" + gemm_source(base, a.dtype);
   });
 
   struct {
@@ -194,25 +249,12 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   std::ostringstream d;
   d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : " mfma 256x256 tiles");
   if (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge) d << " edge";
+  if (bt) d << " B^T";
   if (split) d << " slices=" << slices;
   r.detail = d.str();
   record(std::move(r), k, bytes);
   if (split) {
-    ReduceJob fold;
-    Instr ld;
-    ld.op = Op::Load;
-    ld.dtype = DType::F32;
-    ld.operand = 0;
-    fold.pre.ins.push_back(ld);
-    fold.pre.result = 0;
-    ld.dtype = a.dtype;
-    fold.post.ins.push_back(ld);
-    fold.post.result = 0;
-    fold.operands = {out};
-    fold.axis = 0;
-    fold.rop = ReduceOp::Sum;
-    fold.fold_dtype = a.dtype;
-    return launch_reduce(fold);
+    return fold_slices(out);
   }
   return out;
 }
