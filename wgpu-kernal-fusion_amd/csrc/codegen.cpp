@@ -48,6 +48,34 @@ bool uses_trig(const Program& p, MathPolicy policy) {
   return false;
 }
 
+// An exact transcendental op with an f16 result is evaluated in f64 and rounded to f16 ONCE.  The
+// compiler's f64 -> f16 conversion is a long integer sequence, so the common case goes f64 -> f32 -> f16
+// and only a value whose f32 rounding lies within an f32 ulp of an f16 rounding boundary (where the two
+// roundings could differ from one) takes the direct conversion.
+const char* const kRoundH =
+    "static __device__ __forceinline__ _Float16 wkf_round_h(double d) {\n"
+    "  const float y = (float)d;\n"
+    "  const _Float16 lo = (_Float16)(y * 0x1.fffffep-1f), hi = (_Float16)(y * 0x1.000002p+0f);\n"
+    "  if (__builtin_expect(lo == hi, 1)) return lo;\n"
+    "  return (_Float16)d;\n"
+    "}\n";
+
+bool is_transcendental(Op o) {
+  switch (o) {
+    case Op::Load: case Op::AddC: case Op::SubC: case Op::RSubC: case Op::MulC: case Op::DivC: case Op::RDivC: case Op::Sqr:
+    case Op::Neg: case Op::Abs: case Op::Cast: case Op::Add: case Op::Sub: case Op::Mul: case Op::Div: case Op::Sqrt:
+      return false;
+    default:
+      return true;
+  }
+}
+
+bool uses_round_h(const Program& p, MathPolicy policy) {
+  for (size_t i = 0; i < p.ins.size(); i++)
+    if (p.ins[i].dtype == DType::F16 && is_transcendental(p.ins[i].op) && exact_op(p, i, policy)) return true;
+  return false;
+}
+
 const char* lib_fn(Op o) {
   switch (o) {
     case Op::Exp: return "exp";
@@ -72,12 +100,14 @@ const char* lib_fn(Op o) {
 }
 
 // f32 -> f32 call text of a unary math op on the f32 expression `a`.
-std::string math_call(Op o, const std::string& a, bool exact, bool far_variant) {
+// `wide`: the destination is f16, so an exact op yields its f64 value (rounded once by the caller's cast).
+std::string math_call(Op o, const std::string& a, bool exact, bool far_variant, bool wide = false) {
   const std::string f = lib_fn(o);
   if (o == Op::Sqrt || !exact) return f + "f(" + a + ")";  // sqrtf is correctly rounded already
-  if (o == Op::Exp) return "wkf_exp(" + a + ")";
-  if (o == Op::Sin || o == Op::Cos) return "wkf_" + f + (far_variant ? "_far(" + a + ")" : "(" + a + ", far)");
-  return "(float)" + f + "((double)(" + a + "))";  // the library's f64 routine, rounded once
+  const char* d = wide ? "_d" : "";
+  if (o == Op::Exp) return std::string("wkf_exp") + d + "(" + a + ")";
+  if (o == Op::Sin || o == Op::Cos) return "wkf_" + f + (far_variant ? std::string("_far") + d + "(" + a + ")" : std::string(d) + "(" + a + ", far)");
+  return (wide ? "" : "(float)") + f + "((double)(" + a + "))";  // the library's f64 routine, rounded once
 }
 
 // Emits `static __device__ RT name(T0 x0, ..., const float* c[, bool& far])`: one
@@ -122,21 +152,28 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
       case Op::Div: o << a << " / " << b; break;
       case Op::Pow: {
         const bool exact = exact_op(p, i, policy);
-        std::string call = exact ? "(float)pow((double)" + a + ", (double)" + b + ")"
+        std::string call = exact ? std::string(h ? "" : "(float)") + "pow((double)" + a + ", (double)" + b + ")"
                                  : (h ? "powf((float)" + a + ", (float)" + b + ")" : "powf(" + a + ", " + b + ")");
-        o << (h ? "(_Float16)" : "") << call;
+        if (h && exact) o << "wkf_round_h(" << call << ")";
+        else o << (h ? "(_Float16)" : "") << call;
         break;
       }
       default: {
         const bool exact = exact_op(p, i, policy);
+        if (h && exact && in.op == Op::Exp && policy != MathPolicy::Exact) {
+          // an interior exp on f16: correctly rounded through the f32 library with a rare f64 fallback
+          o << "wkf_exp_h((float)" << a << ")";
+          break;
+        }
         if (h && !exact && in.op == Op::Exp) {
           // f16 result: 2^(x log2 e) on the hardware unit (relative error about 2^-21 for any f16 argument,
           // a thousand times finer than the f16 grid); the f32 library's exp would cost more than the loads.
           o << "(_Float16)__builtin_amdgcn_exp2f((float)" << a << " * 0x1.715476p+0f)";
           break;
         }
-        std::string call = math_call(in.op, h ? "(float)" + a : a, exact, far_variant);
-        o << (h ? "(_Float16)" : "") << call;
+        std::string call = math_call(in.op, h ? "(float)" + a : a, exact, far_variant, h);
+        if (h && exact) o << "wkf_round_h(" << call << ")";
+        else o << (h ? "(_Float16)" : "") << call;
       }
     }
     o << ";\n";
@@ -201,6 +238,7 @@ std::string map_tiled_source(const MapSpec& s) {
   std::ostringstream o;
   o << kPrelude;
   if (uses_math(s.prog, s.math)) o << kMath;
+  if (uses_round_h(s.prog, s.math)) o << kRoundH;
   o << "struct Args { void* p[" << N << "]; u32 nwork; u32 shape[" << R << "]; u32 off[" << N << "]; u32 stride[" << N
     << "][" << R << "]; float c[" << NC << "]; };\n";
   std::vector<DType> types;
@@ -304,6 +342,11 @@ std::string map_source(const MapSpec& s) {
     any_trig |= trig.back();
   }
   if (any_math) o << kMath;
+  {
+    bool any_round_h = false;
+    for (const Program* p : progs) any_round_h |= uses_round_h(*p, s.math);
+    if (any_round_h) o << kRoundH;
+  }
   o << "struct Args { void* p[" << N << "]; u32 nwork; u32 shape[" << R << "]; u32 off[" << N << "]; u32 stride[" << N
     << "][" << R << "]; float c[" << NC << "]; };\n";
   std::vector<DType> types;
@@ -495,6 +538,7 @@ std::string reduce_source(const ReduceSpec& s) {
   std::ostringstream o;
   o << kPrelude;
   if (uses_math(s.pre, s.math_pre) || (!raw && uses_math(s.post, s.math_post))) o << kMath;
+  if (uses_round_h(s.pre, s.math_pre) || (!raw && uses_round_h(s.post, s.math_post))) o << kRoundH;
   o << fold_macro(s.rop);
   o << kReduceHelpers;
   o << "struct Args { void* p[" << N + 1 << "]; u32 nrows; u32 n; u32 nvec; u32 oshape[" << std::max(1, Ro)
@@ -790,6 +834,11 @@ std::string row_source(const RowSpec& s) {
   bool math = !s.store_scalars && uses_math(s.final, store_policy);
   for (const auto& st : s.stages) math |= uses_math(st.pre, fold_policy) || uses_math(st.post, store_policy);
   if (math) o << kMath;
+  {
+    bool round_h = !s.store_scalars && uses_round_h(s.final, store_policy);
+    for (const auto& st : s.stages) round_h |= uses_round_h(st.pre, fold_policy) || uses_round_h(st.post, store_policy);
+    if (round_h) o << kRoundH;
+  }
   o << kRowHelpers;
   o << "struct Args { void* p[" << K + NOUT << "]; u32 nrows; u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
     << "]; u32 ostride[" << K + NOUT << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
