@@ -197,6 +197,29 @@ def test_transposed_operands_take_the_tiled_kernel(gpu, dtype):
         assert_ulp(g, w, 2)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+def test_transposed_operands_with_aligned_shapes(gpu, dtype):
+    # the tiled kernel on shapes that are multiples of the vector width, with a per-row scalar operand and sliced views
+    api = HipAPI(gpu)
+    a = data((304, 520), -2, 2, dtype, 25)
+    b = data((520, 304), -2, 2, dtype, 26)
+    c = data((3, 136, 264), -2, 2, dtype, 27)
+    r = data((520,), 0.5, 2, dtype, 28)
+
+    def progs(ta, tb, tc, tr):
+        return [ta.transpose(0, 1) + 1.0,
+                ta.transpose(0, 1) * tb - tb,
+                (ta.transpose(0, 1) + tb) / tr.broadcast([520, 304]),            # one scalar per output row
+                tc.transpose(1, 2) * 2.0,                                        # batch dim in front, partial edge tiles
+                ta.slice([(8, 296), (16, 504)]).transpose(0, 1) * tb.slice([(16, 504), (8, 296)]),
+                ta.transpose(0, 1).exp() + tb]
+
+    got = hip_values_many(progs(api.tensor(a), api.tensor(b), api.tensor(c), api.tensor(r)))
+    want = progs(OTensor(a), OTensor(b), OTensor(c), OTensor(r))
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert_ulp(g, w.to_numpy(), 0, f"program {i}")
+
+
 def test_same_results_under_both_fusion_modes(gpu):
     a, b = data((64, 96), -2, 2, np.float32, 11), data((64, 96), 0.5, 2, np.float32, 12)
     api = HipAPI(gpu)
