@@ -123,13 +123,22 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
   o << "static __device__ " << (far_variant ? "__attribute__((noinline)) " : "__forceinline__ ") << ctype(p.result_dtype())
     << " " << name << (far_variant ? "_far" : "") << "(";
   for (size_t i = 0; i < operand_types.size(); i++) o << ctype(operand_types[i]) << " x" << i << ", ";
-  o << "const float* c" << (trig && !far_variant ? ", bool& far" : "") << ") {\n";
+  if (far_variant) {
+    // constants by value: handing a pointer into the kernel-argument block to a function that is not
+    // inlined makes the compiler copy the whole block to scratch memory and use it from there
+    o << "int";
+    for (size_t i = 0; i < p.consts.size(); i++) o << ", float k" << i;
+    o << ") {\n";
+  } else {
+    o << "const float* c" << (trig ? ", bool& far" : "") << ") {\n";
+  }
   for (size_t i = 0; i < p.ins.size(); i++) {
     const Instr& in = p.ins[i];
     const bool h = in.dtype == DType::F16;
     const char* t = ctype(in.dtype);
     std::string a = "v" + std::to_string(in.a), b = "v" + std::to_string(in.b);
-    std::string k = h ? "(_Float16)c[" + std::to_string(in.cslot) + "]" : "c[" + std::to_string(in.cslot) + "]";
+    const std::string kref = far_variant ? "k" + std::to_string(in.cslot) : "c[" + std::to_string(in.cslot) + "]";
+    std::string k = h ? "(_Float16)" + kref : kref;
     o << "  const " << t << " v" << i << " = ";
     switch (in.op) {
       case Op::Load: o << "x" << in.operand; break;
@@ -179,6 +188,15 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
     o << ";\n";
   }
   o << "  return v" << p.result << ";\n}\n";
+}
+
+// The constant argument(s) of a call to an emitted program: the pointer `base + off` for the ordinary
+// variant, a dummy int followed by the values themselves for the far variant.
+std::string const_args(const Program& p, const std::string& base, int off, bool far_variant) {
+  if (!far_variant) return off ? base + " + " + std::to_string(off) : base;
+  std::string r = "0";
+  for (size_t i = 0; i < p.consts.size(); i++) r += ", " + base + "[" + std::to_string(off + int(i)) + "]";
+  return r;
 }
 
 void emit_program(std::ostringstream& o, const Program& p, const std::string& name,
@@ -302,10 +320,9 @@ std::string map_tiled_source(const MapSpec& s) {
     if (s.crossed[k]) call << "tile" << k << "[tx][ty * " << PER << "u + j], ";
     else call << "s" << k << "[j], ";
   }
-  call << "a.c";
   if (trig) o << "    bool far = false;\n";
-  o << "    " << ctype(s.out.dtype) << " v = wkf_expr(" << call.str() << (trig ? ", far" : "") << ");\n";
-  if (trig) o << "    if (__builtin_expect(far, 0)) v = wkf_expr_far(" << call.str() << ");\n";
+  o << "    " << ctype(s.out.dtype) << " v = wkf_expr(" << call.str() << "a.c" << (trig ? ", far" : "") << ");\n";
+  if (trig) o << "    if (__builtin_expect(far, 0)) v = wkf_expr_far(" << call.str() << const_args(s.prog, "a.c", 0, true) << ");\n";
   o << "    if (b_live && aa < A) " << ptr(N - 1) << "[base" << N - 1 << " + aa * a.stride[" << N - 1 << "][" << TA
     << "] + bb * a.stride[" << N - 1 << "][" << TB << "]] = v;\n";
   o << "  }\n}\n";
@@ -418,9 +435,7 @@ std::string map_source(const MapSpec& s) {
           if (is_vec_load(k)) o << "[" << e << "]";
           o << ", ";
         }
-        o << "a.c";
-        if (coff[q]) o << " + " << coff[q];
-        o << (trig[q] && !far_variant ? ", far" : "") << ");\n";
+        o << const_args(*progs[q], "a.c", coff[q], far_variant) << (trig[q] && !far_variant ? ", far" : "") << ");\n";
       }
     }
   };
@@ -568,8 +583,9 @@ std::string reduce_source(const ReduceSpec& s) {
   // A post chain with sin / cos runs once per output, so it simply takes the far variant.
   auto store_value = [&](const std::string& acc) {
     if (raw) return acc;
-    return std::string(uses_trig(s.post, s.math_post) ? "wkf_post_far((" : "wkf_post((") + ctype(s.fold_dtype) + ")" + acc +
-           ", a.c + " + std::to_string(NCpre) + ")";
+    const bool post_far = uses_trig(s.post, s.math_post);
+    return std::string(post_far ? "wkf_post_far((" : "wkf_post((") + ctype(s.fold_dtype) + ")" + acc + ", " +
+           const_args(s.post, "a.c", NCpre, post_far) + ")";
   };
   std::string out_ptr = std::string("((") + ctype(raw ? DType::F32 : s.out_dtype) + "*)a.p[" + std::to_string(N) + "])";
 
@@ -609,7 +625,7 @@ std::string reduce_source(const ReduceSpec& s) {
           }
           o << ", ";
         }
-        o << "a.c" << (trig && !far_variant ? ", far" : "") << ");\n";
+        o << const_args(s.pre, "a.c", 0, far_variant) << (trig && !far_variant ? ", far" : "") << ");\n";
       }
     };
     // loads -> pre on every element -> (rarely) redo through the far variant -> fold
@@ -695,7 +711,7 @@ std::string reduce_source(const ReduceSpec& s) {
               if (wide(k)) o << "[" << e << "]";
               o << ", ";
             }
-            o << "a.c" << (trig && !far_variant ? ", far" : "") << ");\n";
+            o << const_args(s.pre, "a.c", 0, far_variant) << (trig && !far_variant ? ", far" : "") << ");\n";
           }
       };
       values(false, ind);
