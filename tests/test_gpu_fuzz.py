@@ -216,11 +216,14 @@ class Gen:
     def describe(self):
         return "; ".join(f"v{k}={d}" for k, (d, _) in enumerate(self.steps))
 
-    def run(self, make_tensor, T, upto):
+    def run_all(self, make_tensor, T, upto):
         vals = []
         for desc, fn in self.steps[: upto + 1]:
             vals.append(fn(vals, make_tensor, T))
-        return vals[upto]
+        return vals
+
+    def run(self, make_tensor, T, upto):
+        return self.run_all(make_tensor, T, upto)[upto]
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
@@ -239,3 +242,11 @@ def test_random_graphs_are_bit_exact_in_both_fusion_modes(gpu, wkf, seed, dtype)
                 gpu.set_fusion(wkf.FUSION_TREE)
             assert got.shape == want.shape and got.dtype == want.dtype, f"root v{root} mode {mode}: {g.describe()}"
             assert np.array_equal(got, want), f"root v{root} mode {mode} differs from the oracle: {g.describe()}"
+    # the same roots as ONE graph materialised in one pass (shared sub-graphs once, sibling reductions together)
+    vals = g.run_all(api.tensor, api.T, roots[-1])
+    wants = g.run_all(lambda a: OTensor(a), OTensor, roots[-1])
+    if gpu.is_planner:
+        wkf.materialize_many([vals[r] for r in roots])
+        pytest.skip("plan-only device: kernels compiled, nothing computed")
+    for r, sl in zip(roots, wkf.as_slice_many([vals[r] for r in roots])):
+        assert np.array_equal(sl.to_numpy(), wants[r].to_numpy()), f"root v{r} of the joint pass differs: {g.describe()}"
