@@ -463,6 +463,36 @@ def test_composites_small(gpu, mode):
     assert np.allclose(got[4].sum(-1), 1.0, atol=1e-5)
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_composites_on_random_shapes(gpu, seed):
+    # row kernels pick lanes per row and vectors per lane from the shape: odd, prime, tiny and long rows, 1-3 leading dims
+    rng = np.random.default_rng(500 + seed)
+    n = int(rng.choice([1, 2, 3, 7, 8, 30, 64, 100, 128, 255, 384, 1000, 1024, 2040, 4096, 5000, 8192, 12288, 20000]))
+    lead = [int(rng.integers(1, 40)) for _ in range(int(rng.integers(1, 4)))]
+    while np.prod(lead) * n > (1 << 21):
+        lead = lead[:-1] if len(lead) > 1 else [max(1, lead[0] // 2)]
+    shape = tuple(lead) + (n,)
+    x = data(shape, -3, 3, np.float32, 600 + seed)
+    w = data((n,), 0.5, 1.5, np.float32, 700 + seed)
+    api = HipAPI(gpu)
+    x2 = x.reshape(-1, n)
+
+    def progs(tx, tx2, tw):
+        out = [tx.softmax_last_dim(), tx2.layer_norm(tw, 1e-5), tx.silu() * tx, (tx - 1.0).exp().sum(len(shape) - 1),
+               tx.max(len(shape) - 1), tx.sum(0)]
+        return out
+
+    got = hip_values_many(progs(api.tensor(x), api.tensor(x2), api.tensor(w)))
+    want = [t.to_numpy() for t in progs(OTensor(x), OTensor(x2), OTensor(w))]
+    assert np.allclose(got[0], want[0], rtol=1e-5, atol=1e-9), f"softmax {shape}"
+    assert np.allclose(got[1], want[1], rtol=1e-5, atol=1e-7), f"rms norm {shape}"
+    assert_ulp(got[2], want[2], 0, f"silu * x {shape}")  # exp is interior: bit-exact
+    assert np.allclose(got[3], want[3], rtol=1e-5), f"sum(exp(x - 1)) {shape}"
+    assert np.array_equal(got[4], want[4]), f"max {shape}"
+    scale = np.abs(x.astype(np.float64)).sum(0)
+    assert np.all(np.abs(got[5].astype(np.float64) - x.astype(np.float64).sum(0)) <= 1e-5 * scale + 1e-30), f"sum(0) {shape}"
+
+
 # ---- the benchmark configurations at full size ------------------------------------------------------------------------------
 
 def test_config1_fused_unary_chain_full_size(gpu):
