@@ -201,7 +201,7 @@ def build_workloads(w, dev, seeded, which):
 def copy_ceiling(w, dev):
     """Achieved GB/s of a plain device copy kernel (1 GiB read + 1 GiB write), for scale."""
     x = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32))
-    t = x.reshape([1 << 14, 1 << 14])  # reshape = one dense copy kernel
+    t = x.resize([1 << 28])  # resize to the same shape = one dense copy kernel
     wl = Workload("copy", [[t]], 2 * (1 << 30), "GB/s", HBM_PEAK_GBS)
     k = measure_kernels(dev, wl, 10, 3)
     return round(wl.work / k[0]["us"] * 1e-3, 1)
@@ -237,7 +237,7 @@ def plan_only(w):
         return np.zeros(shape, dtype=dtype)
 
     before = dev.module_stats()
-    copy = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32)).reshape([1 << 14, 1 << 14])
+    copy = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32)).resize([1 << 28])
     copy.materialize()
     del copy
     for gname in ("c1", "c2", "c3", "c4", "c5"):

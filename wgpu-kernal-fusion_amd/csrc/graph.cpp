@@ -1296,6 +1296,16 @@ TensorData Resolver::run_resize(const NodeP& n) {
     eb.prog.result = eb.load(resolve(n->a));
   }
   const DType dt = eb.prog.result_dtype();
+  if (is_reshape && st_.fusion == FusionMode::Tree && eb.prog.ins.size() == 1 && eb.prog.ins[0].op == Op::Load &&
+      eb.operands[0].layout.strides == Layout::contiguous_strides(eb.operands[0].layout.shape)) {
+    // Reshaping a tensor that already lies dense in memory is a new layout on the same buffer.  (The reference
+    // always copies, src/resize.rs:131-144; the values are the same and the shared buffer is never written in place.)
+    TensorData view = eb.operands[0];
+    const size_t offset = view.layout.offset;
+    view.layout = Layout::contiguous(n->new_shape);
+    view.layout.offset = offset;
+    return view;
+  }
   if (is_reshape || in_shape == n->new_shape) {
     // reshape (src/resize.rs:131-144): a dense copy in the input's own index order;
     // the contiguous result is then read with the new shape.
