@@ -246,6 +246,14 @@ def test_tree_mode_fuses_pair_wise_trees_and_copies(wkf, planner):
     r = q.rope(cos, sin)
     assert _kinds(r) == ["map"]
     assert "outputs=2" in r.kernels()[0].detail and "operands=6" in r.kernels()[0].detail
+    # a cat that is itself the result: one copy kernel per piece (each fused with what produces the piece), no padding pass
+    c3 = wkf.Tensor.cat([q, q * 2.0, _x(wkf, planner, (5, 8, 16), seed=8)], 0)
+    assert _kinds(c3) == ["map", "map", "map"] and c3.shape() == (9, 8, 16)
+    planner.set_fusion(wkf.FUSION_REFERENCE)
+    try:
+        assert len(_kinds(wkf.Tensor.cat([q, q * 2.0], 0))) == 3  # the reference: resize, the product, slice_assign
+    finally:
+        planner.set_fusion(wkf.FUSION_TREE)
     # pieces of different widths: one kernel per piece
     odd = _x(wkf, planner, (2, 8, 10)).narrow(2, 0, 3)
     assert _kinds(wkf.Tensor.cat([odd, _x(wkf, planner, (2, 8, 5), seed=6)], 2) * _x(wkf, planner, (2, 8, 8), seed=7)) == ["map", "map"]

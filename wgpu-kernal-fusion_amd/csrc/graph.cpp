@@ -1333,7 +1333,77 @@ TensorData Resolver::run_resize(const NodeP& n) {
   return out;
 }
 
+namespace {
+// cat([p0, ..., pk], axis) as Tensor::cat builds it (src/composite/cat.rs:3-41): resize(p0) to the total shape,
+// then one slice_assign per further piece, each filling the next range of `axis`.  Returns the pieces in
+// order when `n` is exactly that and the pieces tile the axis without gaps.
+bool match_cat_chain(const Node* n, std::vector<NodeP>* pieces, size_t* axis) {
+  std::vector<std::pair<size_t, NodeP>> assigned;  // (start on the axis, piece), outermost first
+  int ax = -1;
+  const Node* cur = n;
+  const std::vector<size_t>& total = n->shape;
+  while (cur->kind == NodeKind::SliceAssign) {
+    if (cur->shape != total || cur->ranges.size() != total.size() || cur->b->shape.size() != total.size()) return false;
+    int this_ax = -1;
+    for (size_t d = 0; d < total.size(); d++) {
+      const bool whole = cur->ranges[d] == std::make_pair(size_t(0), total[d]) && cur->b->shape[d] == total[d];
+      if (whole) continue;
+      if (this_ax >= 0) return false;
+      this_ax = int(d);
+    }
+    if (this_ax < 0) return false;  // overwrites everything: not a cat
+    if (ax >= 0 && ax != this_ax) return false;
+    ax = this_ax;
+    if (cur->ranges[ax].second - cur->ranges[ax].first != cur->b->shape[ax]) return false;
+    assigned.push_back({cur->ranges[ax].first, cur->b});
+    cur = cur->a.get();
+  }
+  if (cur->kind != NodeKind::Resize || ax < 0 || cur->new_shape != total || cur->fill_shape != cur->a->shape ||
+      cur->a->shape.size() != total.size())
+    return false;
+  for (size_t d = 0; d < total.size(); d++)
+    if (int(d) != ax && cur->a->shape[d] != total[d]) return false;
+  pieces->clear();
+  pieces->push_back(cur->a);
+  size_t at = cur->a->shape[ax];
+  for (size_t i = assigned.size(); i-- > 0;) {
+    if (assigned[i].first != at) return false;
+    pieces->push_back(assigned[i].second);
+    at += assigned[i].second->shape[ax];
+  }
+  if (at != total[ax]) return false;
+  *axis = size_t(ax);
+  return true;
+}
+}  // namespace
+
 TensorData Resolver::run_slice_assign(const NodeP& n) {
+  if (st_.fusion == FusionMode::Tree) {
+    // A whole cat: every piece is written once, straight into its range of a fresh buffer -- no zero fill of
+    // the padded tensor and no read-back (the reference pads, copies and then assigns piece by piece).
+    std::vector<NodeP> pieces;
+    size_t axis = 0;
+    if (match_cat_chain(n.get(), &pieces, &axis)) {
+      TensorData out = alloc(n->shape, n->dtype, false);
+      size_t at = 0;
+      for (const NodeP& piece : pieces) {
+        const size_t len = piece->shape[axis];
+        if (len > 0) {
+          ExprBuilder eb;
+          eb.prog.result = build(eb, piece, pairwise_budget_for_map());
+          if (eb.prog.result_dtype() != n->dtype) invalid("cat: dtype mismatch");
+          std::vector<std::pair<size_t, size_t>> r;
+          for (size_t d = 0; d < n->shape.size(); d++)
+            r.push_back(d == axis ? std::make_pair(at, at + len) : std::make_pair(size_t(0), n->shape[d]));
+          TensorData view = out;
+          view.layout = out.layout.slice(r);
+          launch_map(eb.prog, eb.operands, view, false);
+        }
+        at += len;
+      }
+      return out;
+    }
+  }
   TensorData target = resolve(n->a);
   if (!target.owned() || target.layout.allocation_overlaps()) {
     // The reference writes into the target's buffer whoever else holds it
