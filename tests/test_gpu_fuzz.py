@@ -232,6 +232,14 @@ def test_random_graphs_are_bit_exact_in_both_fusion_modes(gpu, wkf, seed, dtype)
     g = Gen(1000 * seed + (7 if dtype == np.float16 else 0), dtype).build(14)
     api = HipAPI(gpu)
     roots = list(range(len(g.steps)))[-4:]
+    if gpu.is_planner:  # the run that only fills the kernel cache: plan everything this test launches, compute nothing
+        for root in roots:
+            for mode in (wkf.FUSION_TREE, wkf.FUSION_REFERENCE):
+                gpu.set_fusion(mode)
+                try:
+                    g.run(api.tensor, api.T, root).materialize()
+                finally:
+                    gpu.set_fusion(wkf.FUSION_TREE)
     for root in roots:
         want = g.run(lambda a: OTensor(a), OTensor, root).to_numpy()
         for mode in (wkf.FUSION_TREE, wkf.FUSION_REFERENCE):
