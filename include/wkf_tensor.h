@@ -154,6 +154,20 @@ int wkf_tensor_graphvis(const wkf_tensor* t, char* out, size_t cap, size_t* need
 /* The generated HIP source of a kernel signature seen by this process (for inspection and tests). */
 int wkf_kernel_source(const char* signature, char* out, size_t cap, size_t* needed);
 
+/* Layout, src/layout.rs:33-94: the view algebra in elements (offset, shape[rank], strides[rank]) as plain host
+ * functions; nothing here touches a device.
+ * wkf_layout_contiguous  = Layout::contiguous (:41-48): writes the row-major strides of `shape`.
+ * wkf_layout_is_contiguous = Layout::is_contiguous (:58-60): *out = 1 when offset == 0 and the strides are the
+ *   row-major ones of the shape, else 0 (so a slice of one element out of a [2,3] tensor is NOT contiguous).
+ * wkf_layout_slice       = Layout::slice (:62-71) with ranges [begin[d], end[d]): the new offset and shape; the
+ *   strides stay as they are.  end < begin or end > shape is WKF_ERR_INVALID_ARG (the reference's Range::len
+ *   would give 0 for the former and it never checks the latter; a layout that points outside its buffer is
+ *   refused here instead of at the kernel). */
+int wkf_layout_contiguous(int rank, const size_t* shape, size_t* strides_out);
+int wkf_layout_is_contiguous(int rank, size_t offset, const size_t* shape, const size_t* strides, int* out);
+int wkf_layout_slice(int rank, size_t offset, const size_t* shape, const size_t* strides, const size_t* begin,
+                     const size_t* end, size_t* offset_out, size_t* shape_out);
+
 /* Tensor::as_slice, src/tensor.rs:533-554: materialise, download the WHOLE
  * buffer, and keep the layout so that strided views are decoded on the host
  * (TensorSlice, src/tensor.rs:669-855). */

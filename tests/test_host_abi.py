@@ -110,6 +110,40 @@ def test_misuse_returns_status_codes(wkf, planner):
         wkf.Device.new(99)
 
 
+def test_layout_view_algebra(wkf, planner):
+    # test_contiguous, src/layout.rs:96-102
+    layout = wkf.Layout.contiguous([2, 3])
+    assert (layout.offset(), layout.shape(), layout.strides(), layout.rank()) == (0, (2, 3), (3, 1), 2)
+    assert layout.is_contiguous()
+    assert not layout.slice([range(0, 1), range(0, 1)]).is_contiguous()   # strides (3, 1) are not those of a [1, 1] tensor
+    assert not layout.slice([range(1, 2), range(0, 3)]).is_contiguous()   # offset 3
+    # slice keeps the strides, moves the offset and takes the range lengths as the shape (src/layout.rs:15-31,62-71)
+    cube = wkf.Layout.contiguous([4, 5, 6])
+    assert cube.strides() == (30, 6, 1)
+    view = cube.slice([(1, 3), (2, 5), (0, 6)])
+    assert (view.offset(), view.shape(), view.strides()) == (30 + 12, (2, 3, 6), (30, 6, 1))
+    again = view.slice([(1, 2), (1, 3), (4, 6)])                             # ranges are relative to the view
+    assert (again.offset(), again.shape()) == (42 + 30 + 6 + 4, (1, 2, 2))
+    # whole-range slices of a contiguous layout stay contiguous; a leading-dimension prefix does too
+    assert cube.slice([(0, 4), (0, 5), (0, 6)]).is_contiguous()
+    assert cube.slice([(0, 2), (0, 5), (0, 6)]).is_contiguous()
+    assert not cube.slice([(0, 4), (0, 4), (0, 6)]).is_contiguous()
+    # from_parts takes anything; transposed and broadcast strides are not contiguous, rank 0 is
+    assert not wkf.Layout.from_parts(0, [3, 2], [1, 3]).is_contiguous()
+    assert not wkf.Layout.from_parts(0, [2, 3], [0, 1]).is_contiguous()
+    assert wkf.Layout.contiguous([]).is_contiguous() and wkf.Layout.contiguous([]).rank() == 0
+    assert wkf.Layout.contiguous([7]).strides() == (1,)
+    # the layouts the library hands out are these: a sliced tensor's view has the layout Layout::slice gives
+    t = wkf.Tensor.new(planner, np.arange(24, dtype=np.float32).reshape(4, 6))
+    got = t.slice([(1, 3), (2, 5)]).as_slice()
+    want = wkf.Layout.contiguous([4, 6]).slice([(1, 3), (2, 5)])
+    assert (got.offset, got.shape, got.strides) == (want.offset(), want.shape(), want.strides())
+    for bad in ([(0, 5), (0, 5), (0, 6)], [(3, 2), (0, 5), (0, 6)], [(0, 4), (0, 5)]):
+        with pytest.raises(wkf.WkfError) as e:
+            cube.slice(bad)
+        assert e.value.code == wkf.ERR_INVALID_ARG
+
+
 def test_hiprtc_failure_is_reported_with_the_log(wkf, planner):
     lib = wkf.load()
     k = ctypes.c_void_p()

@@ -22,6 +22,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libwkf_hip.so")
 
 F32, F16 = 0, 1
+ERR_HIP, ERR_HIPRTC, ERR_INVALID_ARG, ERR_OOM, ERR_NO_DEVICE, ERR_UNSUPPORTED = 1, 2, 3, 4, 5, 6
 FUSION_REFERENCE, FUSION_TREE = 0, 1
 
 OP_ADD_CONST, OP_SUB_CONST, OP_CONST_SUB, OP_MUL_CONST, OP_DIV_CONST, OP_CONST_DIV = range(6)
@@ -48,6 +49,7 @@ EXPORTS = [
     "wkf_tensor_arange", "wkf_tensor_materialize", "wkf_tensor_kernel_count", "wkf_tensor_kernel_info",
     "wkf_kernel_source", "wkf_tensor_graphvis", "wkf_tensor_materialize_many", "wkf_tensor_as_slice_many", "wkf_tensor_as_slice", "wkf_slice_free", "wkf_slice_rank", "wkf_slice_dtype",
     "wkf_slice_layout", "wkf_slice_data", "wkf_slice_get",
+    "wkf_layout_contiguous", "wkf_layout_is_contiguous", "wkf_layout_slice",
 ]
 
 
@@ -129,6 +131,10 @@ def load():
     lib.wkf_slice_dtype.argtypes = [c_void_p]
     lib.wkf_slice_layout.argtypes = [c_void_p, POINTER(c_size_t), POINTER(c_size_t), POINTER(c_size_t)]
     lib.wkf_slice_data.argtypes = [c_void_p, POINTER(c_size_t)]
+    lib.wkf_layout_contiguous.argtypes = [c_int, POINTER(c_size_t), POINTER(c_size_t)]
+    lib.wkf_layout_is_contiguous.argtypes = [c_int, c_size_t, POINTER(c_size_t), POINTER(c_size_t), POINTER(c_int)]
+    lib.wkf_layout_slice.argtypes = [c_int, c_size_t, POINTER(c_size_t), POINTER(c_size_t), POINTER(c_size_t),
+                                     POINTER(c_size_t), POINTER(c_size_t), POINTER(c_size_t)]
     lib.wkf_slice_get.argtypes = [c_void_p, POINTER(c_size_t), POINTER(c_float)]
     lib.wkf_device_create.argtypes = [c_int, POINTER(c_void_p)]
     lib.wkf_device_create_planner.argtypes = [POINTER(c_void_p)]
@@ -178,6 +184,49 @@ def _sizes(values):
 
 
 _NP = {F32: np.float32, F16: np.float16}
+
+
+class Layout:
+    """Layout (src/layout.rs:33-94): offset, shape and strides of a view, in elements."""
+
+    def __init__(self, offset, shape, strides):  # Layout::from_parts, src/layout.rs:50-56
+        self._offset, self._shape, self._strides = int(offset), tuple(int(v) for v in shape), tuple(int(v) for v in strides)
+        if len(self._shape) != len(self._strides):
+            raise ValueError("shape and strides differ in rank")
+
+    from_parts = classmethod(lambda cls, offset, shape, strides: cls(offset, shape, strides))
+
+    @classmethod
+    def contiguous(cls, shape):  # src/layout.rs:41-48
+        strides = _sizes([0] * len(shape))
+        _check(load().wkf_layout_contiguous(len(shape), _sizes(shape), strides))
+        return cls(0, shape, [strides[i] for i in range(len(shape))])
+
+    def is_contiguous(self):  # src/layout.rs:58-60
+        out = c_int()
+        _check(load().wkf_layout_is_contiguous(self.rank(), self._offset, _sizes(self._shape), _sizes(self._strides), byref(out)))
+        return bool(out.value)
+
+    def slice(self, ranges):  # src/layout.rs:62-71; ranges = [(begin, end), ...] or Python slices / ranges
+        spans = [(r.start, r.stop) if isinstance(r, (slice, range)) else tuple(r) for r in ranges]
+        if len(spans) != self.rank():
+            raise WkfError(ERR_INVALID_ARG, "slice: one range per dimension is required")
+        off, shape = c_size_t(), _sizes([0] * self.rank())
+        _check(load().wkf_layout_slice(self.rank(), self._offset, _sizes(self._shape), _sizes(self._strides),
+                                       _sizes([b for b, _ in spans]), _sizes([e for _, e in spans]), byref(off), shape))
+        return Layout(off.value, [shape[i] for i in range(self.rank())], self._strides)
+
+    def rank(self):
+        return len(self._shape)
+
+    def shape(self):
+        return self._shape
+
+    def strides(self):
+        return self._strides
+
+    def offset(self):
+        return self._offset
 
 
 class Device:

@@ -870,6 +870,49 @@ int wkf_tensor_as_slice(wkf_tensor* t, wkf_slice** out) {
 }
 
 void wkf_slice_free(wkf_slice* s) { delete s; }
+namespace {
+Layout layout_from(int rank, size_t offset, const size_t* shape, const size_t* strides, const char* who) {
+  if (rank < 0 || (rank > 0 && (!shape || !strides))) invalid(std::string(who) + ": bad rank / shape / strides");
+  Layout l;
+  l.offset = offset;
+  l.shape.assign(shape, shape + rank);
+  l.strides.assign(strides, strides + rank);
+  return l;
+}
+}  // namespace
+
+int wkf_layout_contiguous(int rank, const size_t* shape, size_t* strides_out) {
+  return guarded([&] {
+    if (rank < 0 || (rank > 0 && (!shape || !strides_out))) invalid("wkf_layout_contiguous: bad rank / shape");
+    const auto st = Layout::contiguous_strides(std::vector<size_t>(shape, shape + rank));
+    for (int d = 0; d < rank; d++) strides_out[d] = st[d];
+  });
+}
+
+int wkf_layout_is_contiguous(int rank, size_t offset, const size_t* shape, const size_t* strides, int* out) {
+  return guarded([&] {
+    need(out, "wkf_layout_is_contiguous");
+    *out = layout_from(rank, offset, shape, strides, "wkf_layout_is_contiguous").is_contiguous() ? 1 : 0;
+  });
+}
+
+int wkf_layout_slice(int rank, size_t offset, const size_t* shape, const size_t* strides, const size_t* begin,
+                     const size_t* end, size_t* offset_out, size_t* shape_out) {
+  return guarded([&] {
+    const Layout l = layout_from(rank, offset, shape, strides, "wkf_layout_slice");
+    if (rank > 0 && (!begin || !end || !shape_out)) invalid("wkf_layout_slice: missing ranges / output");
+    need(offset_out, "wkf_layout_slice");
+    std::vector<std::pair<size_t, size_t>> ranges;
+    for (int d = 0; d < rank; d++) {
+      if (end[d] < begin[d] || end[d] > l.shape[d]) invalid("wkf_layout_slice: range outside the shape");
+      ranges.emplace_back(begin[d], end[d]);
+    }
+    const Layout r = l.slice(ranges);
+    *offset_out = r.offset;
+    for (int d = 0; d < rank; d++) shape_out[d] = r.shape[d];
+  });
+}
+
 int wkf_slice_rank(const wkf_slice* s) { return s ? int(s->layout.rank()) : -1; }
 int wkf_slice_dtype(const wkf_slice* s) { return s ? int(s->dtype) : -1; }
 
