@@ -94,7 +94,9 @@ int wkf_tensor_cast(const wkf_tensor* t, int dtype, wkf_tensor** out);
 int wkf_tensor_binary_op(const wkf_tensor* a, const wkf_tensor* b, int op, wkf_tensor** out);
 /* Sum::sum / Max::max / Min::min / Product::product over `axis`; rank drops by one. */
 int wkf_tensor_reduce(const wkf_tensor* t, int reduce_op, size_t axis, wkf_tensor** out);
-/* Tensor::mat_mul, src/matmul.rs:25-29: rank 2, same dtype, [M,K] x [K,N]. */
+/* Tensor::mat_mul, src/matmul.rs:25-29: rank 2, same dtype, [M,K] x [K,N].  Beyond the reference (whose mat_mul
+ * is rank 2 only): operands of equal rank > 2 are a batch, [..., M, K] x [..., K, N] -> [..., M, N] with equal
+ * leading dimensions (at most 65535 matrices), one launch for all of them. */
 int wkf_tensor_mat_mul(const wkf_tensor* a, const wkf_tensor* b, wkf_tensor** out);
 
 /* Zero-copy views, src/map_layout.rs:42-98. */

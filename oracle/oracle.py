@@ -164,9 +164,10 @@ class OTensor:
     # -- matmul: the textbook product the reference's own test checks against
     # (ndarray `dot`, src/matmul.rs:268-318); accumulated in float64, rounded once.
     def mat_mul(self, o):
-        if self.a.ndim != 2 or o.a.ndim != 2:
-            raise ValueError("mat_mul: rank 2 only")
-        if self.a.shape[1] != o.a.shape[0]:
+        # rank 2 in the reference; equal leading dimensions are a batch of independent products (this library's extension)
+        if self.a.ndim < 2 or o.a.ndim != self.a.ndim or self.a.shape[:-2] != o.a.shape[:-2]:
+            raise ValueError("mat_mul: operands must have the same rank (2 or more) and the same batch dimensions")
+        if self.a.shape[-1] != o.a.shape[-2]:
             raise ValueError("mat_mul: inner dimensions differ")  # src/matmul.rs:194
         return self._like(self._x() @ o._x())
 

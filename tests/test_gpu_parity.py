@@ -612,6 +612,39 @@ def test_mat_mul_with_a_transposed_weight(gpu, m, n, k, dtype, tol):
     gemm_check(got, a, np.ascontiguousarray(w.T), tol)
 
 
+# (batch dimensions, m, n, k, B given as a transposed view): attention-like products, ragged ones, tiny ones
+BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3), 17, 33, 65, False), ((5,), 3, 5, 7, False),
+                ((8,), 512, 512, 128, True), ((8,), 512, 128, 512, False), ((2, 2), 300, 264, 72, True), ((6,), 1, 384, 128, True),
+                ((3,), 20, 100, 64, True), ((1,), 256, 512, 128, False), ((70,), 64, 64, 32, False)]
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
+@pytest.mark.parametrize("lead,m,n,k,bt", BATCH_SHAPES, ids=[f"{'x'.join(map(str, l))}_{m}x{n}x{k}{'_bt' if t else ''}" for l, m, n, k, t in BATCH_SHAPES])
+def test_batched_mat_mul(gpu, lead, m, n, k, bt, dtype, tol):
+    # [..., M, K] x [..., K, N]: every matrix of the batch against its own float64 product; one launch for the batch
+    rng = np.random.default_rng(sum(lead) * 31 + m * 1000003 + n * 1009 + k)
+    a = rng.standard_normal(lead + (m, k)).astype(dtype)
+    b = rng.standard_normal(lead + ((n, k) if bt else (k, n))).astype(dtype)
+    api = HipAPI(gpu)
+    tb = api.tensor(b)
+    R = len(lead) + 2
+    prod = api.tensor(a).mat_mul(tb.transpose(R - 2, R - 1) if bt else tb)
+    got = hip_values(prod)
+    assert got.dtype == dtype and got.shape == lead + (m, n)
+    dense_b = np.swapaxes(b, -1, -2) if bt else b
+    for idx in np.ndindex(*lead):
+        gemm_check(got[idx], a[idx], np.ascontiguousarray(dense_b[idx]), tol)
+    launches = [kk for kk in prod.kernels() if kk.kind == "gemm"]
+    assert len(launches) == 1
+    # and the same numbers as one product at a time
+    first = tuple(0 for _ in lead)
+    alone = hip_values(api.tensor(a[first]).mat_mul(api.tensor(np.ascontiguousarray(dense_b[first]))))
+    if not bt:
+        assert np.array_equal(alone, got[first])
+    else:
+        gemm_check(alone, a[first], np.ascontiguousarray(dense_b[first]), tol)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
 def test_mat_mul_identities_and_views(gpu, dtype):
     rng = np.random.default_rng(23)

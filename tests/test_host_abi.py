@@ -381,6 +381,31 @@ def test_mat_mul_kernel_choice(wkf, planner):
         planner.set_fusion(wkf.FUSION_TREE)
 
 
+def test_batched_mat_mul_is_one_launch(wkf, planner):
+    # beyond the reference (rank 2 only, src/matmul.rs:25-29): equal leading dimensions are a batch
+    q = _x(wkf, planner, (8, 512, 128), np.float16)
+    k = _x(wkf, planner, (8, 512, 128), np.float16, seed=1)
+    scores = q.mat_mul(k.transpose(1, 2))                      # q k^T per head: k is read as it lies
+    assert scores.shape() == (8, 512, 512) and _kinds(scores) == ["gemm"]
+    assert scores.kernels()[0].detail.endswith("B^T batch=8") and "|bt" in scores.kernels()[0].signature
+    v = _x(wkf, planner, (8, 512, 128), np.float16, seed=2)
+    out = scores.softmax_last_dim().mat_mul(v)
+    assert out.shape() == (8, 512, 128) and _kinds(out) == ["gemm", "row", "gemm"]
+    assert out.kernels()[2].detail.endswith("edge batch=8")    # n = 128 is half a tile: the edge kernel
+    r4 = _x(wkf, planner, (2, 3, 17, 33), np.float32).mat_mul(_x(wkf, planner, (2, 3, 33, 5), np.float32, seed=1))
+    assert r4.shape() == (2, 3, 17, 5) and _kinds(r4) == ["gemm"] and r4.kernels()[0].detail.endswith("generic batch=6")
+    # the same binaries as a single product: no new module for the batch
+    before = planner.module_stats()
+    _x(wkf, planner, (3, 256, 64), np.float16).mat_mul(_x(wkf, planner, (3, 64, 256), np.float16, seed=1)).materialize()
+    _x(wkf, planner, (256, 64), np.float16).mat_mul(_x(wkf, planner, (64, 256), np.float16, seed=1)).materialize()
+    after = planner.module_stats()
+    assert (after["compiled"] + after["disk_hits"]) - (before["compiled"] + before["disk_hits"]) <= 1
+    for bad_a, bad_b in (((2, 4, 8), (3, 8, 4)), ((2, 4, 8), (8, 4)), ((2, 4, 8), (2, 7, 4)), ((8,), (8,))):
+        with pytest.raises(wkf.WkfError) as e:
+            _x(wkf, planner, bad_a, np.float32).mat_mul(_x(wkf, planner, bad_b, np.float32, seed=1))
+        assert e.value.code == wkf.ERR_INVALID_ARG
+
+
 def test_one_binary_serves_every_size_and_constant(wkf, planner):
     before = planner.module_stats()
     t1 = (_x(wkf, planner, (256, 256)) * 3.0) + 5.0

@@ -66,20 +66,37 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // no fusion on either side (src/compute_graph/resolve.rs:138-154)
   TensorData a = resolve(n->a);
   TensorData b = resolve(n->b);
-  if (a.layout.rank() != 2 || b.layout.rank() != 2) invalid("mat_mul: both operands must have rank 2");
+  const size_t R = a.layout.rank();
+  if (R < 2 || b.layout.rank() != R) invalid("mat_mul: operands must have the same rank, 2 or (for a batch) more");
   if (a.dtype != b.dtype) invalid("mat_mul: operand dtypes differ");
-  const size_t M = a.layout.shape[0], K = a.layout.shape[1], N = b.layout.shape[1];
-  if (b.layout.shape[0] != K) invalid("mat_mul: inner dimensions differ");  // src/matmul.rs:194
+  // leading dimensions are a batch of independent products (no counterpart in the reference, whose mat_mul is rank 2)
+  size_t batch = 1;
+  std::vector<size_t> out_shape;
+  for (size_t d = 0; d + 2 < R; d++) {
+    if (a.layout.shape[d] != b.layout.shape[d]) invalid("mat_mul: batch dimensions differ");
+    batch *= a.layout.shape[d];
+    out_shape.push_back(a.layout.shape[d]);
+  }
+  const size_t M = a.layout.shape[R - 2], K = a.layout.shape[R - 1], N = b.layout.shape[R - 1];
+  if (b.layout.shape[R - 2] != K) invalid("mat_mul: inner dimensions differ");  // src/matmul.rs:194
+  out_shape.push_back(M);
+  out_shape.push_back(N);
   // The reference kernel ignores strides and offsets (src/matmul.rs:96-103), which is only
   // right for contiguous operands; a view is copied into a dense buffer first.
   a = make_contiguous(a);
-  // ... except B = transpose(W) of a dense W[N][K] (x * W^T, the linear-layer form): the MFMA kernels read
-  // it as it lies (k contiguous), when its rows are 16-byte aligned and the problem is worth a tile.
-  const bool b_is_t = st_.fusion == FusionMode::Tree && b.layout.offset == 0 && K > 1 && N > 1 && b.layout.strides[0] == 1 &&
-                      b.layout.strides[1] == K;
+  // ... except B = transpose(W) of a dense W[N][K] (x * W^T, the linear-layer form; q * k^T per head in a
+  // batch): the MFMA kernels read it as it lies (k contiguous), when its rows are 16-byte aligned and the
+  // problem is worth a tile.
+  bool b_is_t = st_.fusion == FusionMode::Tree && K > 1 && N > 1;
+  if (b_is_t) {
+    Layout w = b.layout;  // the last two dimensions swapped back: dense exactly when b is such a transpose
+    std::swap(w.shape[R - 2], w.shape[R - 1]);
+    std::swap(w.strides[R - 2], w.strides[R - 1]);
+    b_is_t = w.is_contiguous();
+  }
   const size_t V = a.dtype == DType::F16 ? 8 : 4;
   // ... and with up to 32 rows of A (decode) W is streamed once, straight into MFMA operands
-  const bool skinny_bt = b_is_t && M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);
+  const bool skinny_bt = batch == 1 && b_is_t && M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);
   bool bt = false;
   if (skinny_bt) {
     // handled below
@@ -88,7 +105,8 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   } else {
     b = make_contiguous(b);
   }
-  if (M == 0 || N == 0) return alloc({M, N}, a.dtype, false);
+  if (M == 0 || N == 0 || batch == 0) return alloc(out_shape, a.dtype, false);
+  if (batch > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: more than 65535 matrices in a batch");
   if (M > 0xffffffffull || N > 0xffffffffull || K > 0xffffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: dimension does not fit 32 bits");
   auto fold_slices = [&](const TensorData& part) {
     // adds the f32 partial sums of the K slices ([S][M][N]) and rounds to the tensor dtype
@@ -144,7 +162,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   }
   // A handful of rows (decode): reading B once is all the work -> the bandwidth kernel, K cut into slices
   // across the grid, then one reduce launch that adds the slices and rounds to the tensor dtype.
-  if (st_.fusion == FusionMode::Tree && !bt && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
+  if (st_.fusion == FusionMode::Tree && batch == 1 && !bt && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
     const size_t esize = dtype_size(a.dtype);
     const size_t colblocks = (N + 256 * V - 1) / (256 * V);
     size_t S = (1024 + colblocks - 1) / colblocks;
@@ -194,7 +212,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // (f32 partial sums per slice, then one reduce launch), as long as the partial sums stay below
   // the bytes of A and B.
   size_t slices = 1, kchunk = 0;
-  if (mfma && st_.fusion == FusionMode::Tree) {
+  if (mfma && batch == 1 && st_.fusion == FusionMode::Tree) {
     wkf_props props;
     if (wkf_device_props(dev_, &props) != WKF_OK) throw Error(WKF_ERR_HIP, wkf_last_error());
     const size_t cus = size_t(std::max(1, props.compute_units));
@@ -211,7 +229,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     }
   }
   const bool split = slices > 1;
-  TensorData out = split ? alloc({slices, M, N}, DType::F32, false) : alloc({M, N}, a.dtype, false);
+  TensorData out = split ? alloc({slices, M, N}, DType::F32, false) : alloc(out_shape, a.dtype, false);
   std::string sig = gemm_signature(kind, a.dtype);
   if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
   if (bt) sig += "|bt";
@@ -246,11 +264,13 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.grid[0] = uint32_t(tiles);
     r.grid[1] = uint32_t(slices);
   }
+  r.grid[2] = uint32_t(batch);
   std::ostringstream d;
   d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : " mfma 256x256 tiles");
   if (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge) d << " edge";
   if (bt) d << " B^T";
   if (split) d << " slices=" << slices;
+  if (batch > 1) d << " batch=" << batch;
   r.detail = d.str();
   record(std::move(r), k, bytes);
   if (split) {

@@ -316,10 +316,16 @@ NodeP n_cat(const std::vector<NodeP>& v, size_t dim) {
 }
 
 NodeP n_mat_mul(const NodeP& a, const NodeP& b) {
-  if (a->shape.size() != 2 || b->shape.size() != 2) invalid("mat_mul: both operands must have rank 2");
+  const size_t R = a->shape.size();
+  if (R < 2 || b->shape.size() != R) invalid("mat_mul: operands must have the same rank, 2 or (for a batch) more");
   if (a->dtype != b->dtype) invalid("mat_mul: operand dtypes differ");
-  if (a->shape[1] != b->shape[0]) invalid("mat_mul: inner dimensions differ");  // src/matmul.rs:194
-  NodeP n = make(NodeKind::MatMul, a->dtype, {a->shape[0], b->shape[1]});
+  if (a->shape[R - 1] != b->shape[R - 2]) invalid("mat_mul: inner dimensions differ");  // src/matmul.rs:194
+  std::vector<size_t> shape(a->shape.begin(), a->shape.end() - 2);
+  for (size_t d = 0; d + 2 < R; d++)
+    if (a->shape[d] != b->shape[d]) invalid("mat_mul: batch dimensions differ");
+  shape.push_back(a->shape[R - 2]);
+  shape.push_back(b->shape[R - 1]);
+  NodeP n = make(NodeKind::MatMul, a->dtype, shape);
   n->a = a;
   n->b = b;
   return n;
