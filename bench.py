@@ -265,8 +265,7 @@ def main():
                     help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on ONE GPU (every kernel, no collectives); --gpus must be 1. "
-                 "DESIGN.md says how the path would shard.")
+        sys.exit("bench.py: this build runs on ONE GPU (every kernel, no collectives); --gpus must be 1.")
 
     w = load_package()
     dg_spec = importlib.util.spec_from_file_location("wkf_datagen", os.path.join(ROOT, "wgpu-kernal-fusion_amd", "datagen.py"))

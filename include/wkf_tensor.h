@@ -1,8 +1,8 @@
 /*
  * wkf_tensor.h -- level 1 of the C ABI: the lazy Tensor API of the reference
  * crate (`Tensor<const R, D>`, re-exported by src/lib.rs:1-11) behind opaque C
- * handles.  A Rust `Tensor<R, D>` facade binds these one-to-one (INTEGRATION.md
- * shows the `extern "C"` block); ranks and dtypes are checked at run time where
+ * handles.  A Rust `Tensor<R, D>` facade binds these one-to-one through an
+ * `extern "C"` block; ranks and dtypes are checked at run time where
  * the Rust types check them at compile time.
  *
  * Every op only records a node (src/tensor.rs:179-284); nothing touches the GPU
