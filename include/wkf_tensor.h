@@ -10,6 +10,10 @@
  * panics (shape mismatch, bad axis ...) these return WKF_ERR_INVALID_ARG and
  * leave the message in wkf_last_error().
  *
+ * Threads: graph nodes are immutable and a materialisation keeps its state to itself, so different handles
+ * (also of graphs that share nodes) may be used from different threads at once; the device layer serialises
+ * what reaches the stream.  One handle is for one thread at a time (a materialisation rewrites its launch list).
+ *
  * Paths in comments are relative to the reference checkout.
  */
 #ifndef WKF_TENSOR_H

@@ -144,6 +144,42 @@ def test_layout_view_algebra(wkf, planner):
         assert e.value.code == wkf.ERR_INVALID_ARG
 
 
+def test_a_new_device_starts_with_default_settings(wkf):
+    # per-device state is dropped with the device: a later device (the allocator tends to hand out the same
+    # address again) must not inherit the fusion mode of one that was destroyed
+    for _ in range(8):
+        d = wkf.Device.planner()
+        assert d.fusion() == wkf.FUSION_TREE
+        d.set_fusion(wkf.FUSION_REFERENCE)
+        assert d.fusion() == wkf.FUSION_REFERENCE
+        d.close()
+
+
+def test_graphs_sharing_nodes_resolve_from_several_threads(wkf, planner):
+    # nodes are immutable and a resolution keeps its state to itself, so graphs that share nodes may be
+    # materialised from different threads (one handle per thread); the device layer serialises the launches
+    import threading
+    base = wkf.Tensor.new(planner, np.arange(64 * 64, dtype=np.float32).reshape(64, 64))
+    shared = base.mat_mul(base)
+    roots = [(shared + float(i)).sum(1) for i in range(32)]
+    errors = []
+
+    def work(ts):
+        try:
+            for t in ts:
+                t.materialize()
+                assert [k.kind for k in t.kernels()] == ["gemm", "red_row"]
+        except Exception as e:  # noqa: BLE001
+            errors.append(e)
+
+    threads = [threading.Thread(target=work, args=(roots[i::4],)) for i in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors
+
+
 def test_hiprtc_failure_is_reported_with_the_log(wkf, planner):
     lib = wkf.load()
     k = ctypes.c_void_p()

@@ -126,6 +126,17 @@ struct wkf_timer {
 // Lets the layers above this file leave their message where wkf_last_error() finds it.
 void wkf_set_last_error_(const char* msg) { g_last_error = msg ? msg : ""; }
 
+// The layers above keep per-device state keyed by the handle; they register a function here that forgets a
+// device when it is destroyed, so that a later device at the same address starts clean.
+namespace {
+std::mutex g_hooks_mu;
+std::vector<void (*)(wkf_device*)> g_destroy_hooks;
+}  // namespace
+void wkf_add_destroy_hook_(void (*fn)(wkf_device*)) {
+  std::lock_guard<std::mutex> lock(g_hooks_mu);
+  g_destroy_hooks.push_back(fn);
+}
+
 extern "C" {
 
 const char* wkf_last_error(void) { return g_last_error.c_str(); }
@@ -206,6 +217,14 @@ int wkf_device_trim(wkf_device* dev) {
 
 void wkf_device_destroy(wkf_device* dev) {
   if (!dev) return;
+  {
+    std::vector<void (*)(wkf_device*)> hooks;
+    {
+      std::lock_guard<std::mutex> lock(g_hooks_mu);
+      hooks = g_destroy_hooks;
+    }
+    for (auto fn : hooks) fn(dev);
+  }
   wkf_device_trim(dev);
   for (auto& kv : dev->kernels) {
     if (kv.second->module) hipModuleUnload(kv.second->module);
@@ -301,7 +320,7 @@ void* wkf_buffer_ptr(const wkf_buffer* buf) { return buf ? buf->ptr : nullptr; }
 
 int wkf_buffer_upload(wkf_buffer* buf, size_t offset, const void* src, size_t bytes) {
   if (!buf || (!src && bytes)) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_upload: null argument");
-  if (offset + bytes > buf->capacity) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_upload: range outside the buffer");
+  if (offset > buf->capacity || bytes > buf->capacity - offset) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_upload: range outside the buffer");
   if (!bytes) return WKF_OK;
   wkf_device* dev = buf->dev;
   std::lock_guard<std::recursive_mutex> lock(dev->mu);
@@ -310,6 +329,7 @@ int wkf_buffer_upload(wkf_buffer* buf, size_t offset, const void* src, size_t by
     buf->host_valid = true;
     return WKF_OK;
   }
+  WKF_HIP_CHECK(hipSetDevice(dev->ordinal));
   WKF_HIP_CHECK(hipMemcpyAsync(static_cast<char*>(buf->ptr) + offset, src, bytes, hipMemcpyHostToDevice, dev->stream));
   // The source is pageable host memory the caller may free on return.
   WKF_HIP_CHECK(hipStreamSynchronize(dev->stream));
@@ -318,7 +338,7 @@ int wkf_buffer_upload(wkf_buffer* buf, size_t offset, const void* src, size_t by
 
 int wkf_buffer_download(wkf_buffer* buf, size_t offset, void* dst, size_t bytes) {
   if (!buf || (!dst && bytes)) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_download: null argument");
-  if (offset + bytes > buf->capacity) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_download: range outside the buffer");
+  if (offset > buf->capacity || bytes > buf->capacity - offset) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_download: range outside the buffer");
   if (!bytes) return WKF_OK;
   wkf_device* dev = buf->dev;
   std::lock_guard<std::recursive_mutex> lock(dev->mu);
@@ -328,6 +348,7 @@ int wkf_buffer_download(wkf_buffer* buf, size_t offset, void* dst, size_t bytes)
     memcpy(dst, static_cast<char*>(buf->ptr) + offset, bytes);
     return WKF_OK;
   }
+  WKF_HIP_CHECK(hipSetDevice(dev->ordinal));
   WKF_HIP_CHECK(hipMemcpyAsync(dst, static_cast<char*>(buf->ptr) + offset, bytes, hipMemcpyDeviceToHost, dev->stream));
   WKF_HIP_CHECK(hipStreamSynchronize(dev->stream));
   return WKF_OK;
@@ -366,8 +387,11 @@ int wkf_module_get(wkf_device* dev, const char* signature, const char* hip_sourc
     *out = it->second;
     return WKF_OK;
   }
-  // Disk key: everything that decides the code object's bytes.
+  // Disk key: everything that decides the code object's bytes, the compiler's version included.
   uint64_t h = fnv1a(kCacheVersion, strlen(kCacheVersion));
+  int rtc[2] = {0, 0};
+  if (hiprtcVersion(&rtc[0], &rtc[1]) != HIPRTC_SUCCESS) return fail(WKF_ERR_HIPRTC, "hiprtcVersion failed");
+  h = fnv1a(rtc, sizeof(rtc), h);
   for (int i = 0; i < kNumCompileOptions; i++) h = fnv1a(kCompileOptions[i], strlen(kCompileOptions[i]), h);
   h = fnv1a(entry, strlen(entry), h);
   h = fnv1a(hip_source, strlen(hip_source), h);
@@ -456,6 +480,7 @@ int wkf_module_find(wkf_device* dev, const char* signature, wkf_kernel** out) {
 
 int wkf_module_stats(wkf_device* dev, uint64_t* compiled, uint64_t* disk_hits, uint64_t* mem_hits) {
   if (!dev) return fail(WKF_ERR_INVALID_ARG, "wkf_module_stats: null device");
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
   if (compiled) *compiled = dev->n_compiled;
   if (disk_hits) *disk_hits = dev->n_disk;
   if (mem_hits) *mem_hits = dev->n_mem;
@@ -471,6 +496,7 @@ int wkf_launch(wkf_device* dev, wkf_kernel* kernel, const uint32_t grid[3], cons
   if (dev->planner) return WKF_OK;  // plan-only: nothing runs
   if (!kernel->function) return fail(WKF_ERR_INVALID_ARG, "wkf_launch: kernel has no loaded function");
   std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  WKF_HIP_CHECK(hipSetDevice(dev->ordinal));  // the calling thread may have another device current
   size_t size = arg_bytes;
   void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(args), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                     HIP_LAUNCH_PARAM_END};

@@ -14,6 +14,7 @@ using namespace wkf;
 
 // hip_ffi.cpp owns the thread-local error string; this hook lets the upper layers set it.
 void wkf_set_last_error_(const char* msg);
+void wkf_add_destroy_hook_(void (*fn)(wkf_device*));
 
 struct wkf_tensor {
   wkf_device* dev;
@@ -86,7 +87,14 @@ namespace {
 std::mutex g_settings_mu;
 std::unordered_map<wkf_device*, Settings> g_settings;
 
+void forget_device(wkf_device* dev) {
+  std::lock_guard<std::mutex> lock(g_settings_mu);
+  g_settings.erase(dev);
+}
+
 Settings settings_for(wkf_device* dev) {
+  static const bool hooked = (wkf_add_destroy_hook_(&forget_device), true);
+  (void)hooked;
   std::lock_guard<std::mutex> lock(g_settings_mu);
   auto it = g_settings.find(dev);
   if (it == g_settings.end()) {
@@ -128,6 +136,9 @@ int guarded(F&& f) {
     return WKF_ERR_OOM;
   } catch (const std::exception& e) {
     wkf_set_last_error_(e.what());
+    return WKF_ERR_INVALID_ARG;
+  } catch (...) {
+    wkf_set_last_error_("unknown exception");
     return WKF_ERR_INVALID_ARG;
   }
 }
@@ -876,6 +887,7 @@ int wkf_tensor_as_slice(wkf_tensor* t, wkf_slice** out) {
 }
 
 void wkf_slice_free(wkf_slice* s) { delete s; }
+extern "C++" {
 namespace {
 Layout layout_from(int rank, size_t offset, const size_t* shape, const size_t* strides, const char* who) {
   if (rank < 0 || (rank > 0 && (!shape || !strides))) invalid(std::string(who) + ": bad rank / shape / strides");
@@ -886,6 +898,7 @@ Layout layout_from(int rank, size_t offset, const size_t* shape, const size_t* s
   return l;
 }
 }  // namespace
+}  // extern "C++"
 
 int wkf_layout_contiguous(int rank, const size_t* shape, size_t* strides_out) {
   return guarded([&] {
