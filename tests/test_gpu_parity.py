@@ -493,6 +493,43 @@ def test_composites_on_random_shapes(gpu, seed):
     assert np.all(np.abs(got[5].astype(np.float64) - x.astype(np.float64).sum(0)) <= 1e-5 * scale + 1e-30), f"sum(0) {shape}"
 
 
+RAGGED_ROWS = [(37, 2880, np.float32), (16, 11008, np.float32), (9, 50257, np.float32), (64, 1234, np.float32), (5, 32772, np.float32),
+               (3, 65535, np.float32), (2, 65532, np.float32), (40, 1002, np.float32), (7, 77, np.float32), (11, 5, np.float32),
+               (33, 2880, np.float16), (8, 11004, np.float16), (6, 50257, np.float16), (50, 1234, np.float16), (2, 131070, np.float16)]
+
+
+@pytest.mark.parametrize("rows,n,dtype", RAGGED_ROWS, ids=[f"{r}x{n}_{np.dtype(d).name}" for r, n, d in RAGGED_ROWS])
+def test_row_kernels_on_rows_that_do_not_split_evenly(gpu, rows, n, dtype):
+    # one fused kernel also when the row is not a power-of-two multiple of the vector width: the lanes past the
+    # end of the row are masked in their last vector, and odd or unaligned rows take narrower vectors
+    x = data((rows, n), -3, 3, dtype, rows * 7 + n)
+    w = data((n,), 0.5, 1.5, dtype, n)
+    api = HipAPI(gpu)
+    tx, tw = api.tensor(x), api.tensor(w)
+    ox, ow = OTensor(x), OTensor(w)
+    view = [(1, rows), (1, n - 1)]          # rows of the view start one element into the rows of x
+    progs = [tx.softmax_last_dim(), tx.slice(view).softmax_last_dim(), tx.slice(view).exp().sum(1)]
+    want = [ox.softmax_last_dim().to_numpy(), ox.slice(view).softmax_last_dim().to_numpy(), None]
+    if dtype == np.float32:                  # layer_norm is f32 in the reference (src/composite/rms_norm.rs:8-15)
+        progs.append(tx.layer_norm(tw, 1e-5))
+        want.append(ox.layer_norm(ow, 1e-5).to_numpy())
+    got = hip_values_many(progs)
+    assert [k.kind for k in progs[0].kernels()] == ["row"], [k.detail for k in progs[0].kernels()]
+    rtol = 1e-5 if dtype == np.float32 else 2e-3
+    for i in (0, 1, 3):
+        if i < len(got) and want[i] is not None:
+            assert got[i].shape == want[i].shape
+            assert np.allclose(got[i].astype(np.float64), want[i].astype(np.float64), rtol=rtol, atol=1e-7 if dtype == np.float32 else 1e-6), i
+    assert np.allclose(got[0].astype(np.float64).sum(1), 1.0, atol=1e-5 if dtype == np.float32 else 2e-2)
+    assert np.all(got[0][:, -1] > 0) and np.all(got[1][:, -1] > 0)          # the last element of a row is written
+    ref = np.exp(x[1:, 1:n - 1].astype(np.float64))
+    if dtype == np.float16:
+        ref = ref.astype(np.float16).astype(np.float64)                       # exp is rounded to f16 before the fold
+    with np.errstate(over="ignore"):
+        total = ref.sum(1).astype(dtype).astype(np.float64)                   # a long f16 row overflows to inf, here as there
+    assert np.allclose(got[2].astype(np.float64), total, rtol=1e-5 if dtype == np.float32 else 4e-3)
+
+
 # ---- the benchmark configurations at full size ------------------------------------------------------------------------------
 
 def test_config1_fused_unary_chain_full_size(gpu):

@@ -307,8 +307,9 @@ def test_tree_mode_fuses_pair_wise_trees_and_copies(wkf, planner):
     assert _kinds(ln) == ["row"] and "stages=1" in ln.kernels()[0].detail
     s = _x(wkf, planner, (4, 8, 32)).softmax_last_dim()
     assert _kinds(s) == ["row"] and "stages=2" in s.kernels()[0].detail  # max, sum(exp(x - max)), exp(x - max) / sum
-    # a row length the row kernel does not take (not a multiple of the vector width) falls back to separate kernels
-    assert _kinds(_x(wkf, planner, (8, 30)).softmax_last_dim()) == ["red_row", "red_row", "map"]
+    # a row length that is not a multiple of the 16-byte vector takes narrower vectors in the same kernel
+    odd = _x(wkf, planner, (8, 30)).softmax_last_dim()
+    assert _kinds(odd) == ["row"] and "vec=2" in odd.kernels()[0].detail
     q = _x(wkf, planner, (2, 8, 16))
     cos, sin = _x(wkf, planner, (8, 8), seed=4), _x(wkf, planner, (8, 8), seed=5)
     # rope = ONE kernel: the cats of rotate_half and of the duplicated tables are cut at the seam, both halves of the
@@ -380,6 +381,27 @@ def test_sibling_row_reductions_share_one_pass(wkf, planner):
         planner.set_fusion(wkf.FUSION_TREE)
     with pytest.raises(wkf.WkfError):
         wkf.materialize_many([])
+
+
+def test_row_kernel_takes_rows_that_do_not_split_evenly(wkf, planner):
+    def detail(shape, dtype, f):
+        t = f(_x(wkf, planner, shape, dtype))
+        assert _kinds(t) == ["row"], [k.detail for k in t.kernels()]
+        return t.kernels()[0].detail
+
+    sm = lambda t: t.softmax_last_dim()  # noqa: E731
+    # an even split keeps the exact kernel (no masking) ...
+    assert "ragged" not in detail((8, 4096), np.float32, sm)
+    assert "ragged" not in detail((8, 5120), np.float32, sm)                      # 1280 vectors = 256 lanes x 5
+    # ... anything else gets the widest layout with the tail lanes masked in their last vector
+    assert detail((8, 2880), np.float32, sm).endswith("vec=4 threads_per_row=256 vectors_per_lane=3 stages=2 operands=2 ragged")
+    assert "vec=2" in detail((8, 1002), np.float32, sm) and "vec=1" in detail((8, 50257), np.float32, sm)
+    assert "vec=8" in detail((8, 2880), np.float16, sm) and "vec=4" in detail((8, 11004), np.float16, sm)
+    # rows of a view that start off the vector grid take narrower vectors instead of three kernels
+    assert "vec=1" in detail((8, 4096), np.float32, lambda t: t.slice([(0, 8), (1, 4095)]).softmax_last_dim())
+    # beyond what 1024 lanes hold in registers the reductions and the map run on their own
+    long_rows = _x(wkf, planner, (2, 65537), np.float32).softmax_last_dim()
+    assert _kinds(long_rows) == ["red_row", "red_row", "map"]
 
 
 def test_mat_mul_kernel_choice(wkf, planner):

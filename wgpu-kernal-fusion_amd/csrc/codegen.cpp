@@ -822,6 +822,7 @@ std::string row_signature(const RowSpec& s) {
   for (const auto& st : s.stages) o << "|" << reduce_name(st.rop) << "{" << st.pre.signature() << "}{" << st.post.signature() << "}";
   if (s.store_scalars) o << "|scalars";
   else o << "|final{" << s.final.signature() << "}";
+  if (s.ragged) o << "|ragged";
   return o.str();
 }
 
@@ -856,7 +857,7 @@ std::string row_source(const RowSpec& s) {
     if (round_h) o << kRoundH;
   }
   o << kRowHelpers;
-  o << "struct Args { void* p[" << K + NOUT << "]; u32 nrows; u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
+  o << "struct Args { void* p[" << K + NOUT << "]; u32 nrows; " << (s.ragged ? "u32 nvec; " : "") << "u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
     << "]; u32 ostride[" << K + NOUT << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
   // operand types as every program sees them: the K full operands, then one scalar per earlier stage
   std::vector<DType> types;
@@ -875,6 +876,7 @@ std::string row_source(const RowSpec& s) {
   o << "  const u32 row_raw = blockIdx.x * " << RPB << "u + threadIdx.x / " << T << "u;\n";
   o << "  const bool live = row_raw < a.nrows;\n";
   o << "  const u32 row = live ? row_raw : 0u;\n";
+  if (s.ragged) o << "  const bool last_ok = t + " << (NV - 1) * T << "u < a.nvec;  // this lane's last vector lies inside the row\n";
   if (Ro > 0) {
     o << "  u32 rem = row;\n";
     for (int d = Ro - 1; d > 0; d--) o << "  const u32 i" << d << " = rem % a.oshape[" << d << "]; rem /= a.oshape[" << d << "];\n";
@@ -894,9 +896,11 @@ std::string row_source(const RowSpec& s) {
       o << "  const " << ct << " s" << k << " = q" << k << "[0];\n";
     } else {
       std::string vt = vtype(s.in[k].dtype, V);
-      for (int j = 0; j < NV; j++)
-        o << "  const " << vt << " x" << k << "_" << j << " = __builtin_nontemporal_load((const " << vt << "*)(q" << k << " + (t + "
-          << j * T << "u) * " << V << "u));\n";
+      for (int j = 0; j < NV; j++) {
+        o << "  const " << vt << " x" << k << "_" << j << " = ";
+        if (s.ragged && j == NV - 1) o << "!last_ok ? (" << vt << ")(0) : ";
+        o << "__builtin_nontemporal_load((const " << vt << "*)(q" << k << " + (t + " << j * T << "u) * " << V << "u));\n";
+      }
     }
   }
   auto call_args = [&](int j, int e, int nscalars) {
@@ -916,10 +920,14 @@ std::string row_source(const RowSpec& s) {
     const RowStage& st = s.stages[k];
     o << "  float acc" << k << " = " << seed_text(st.rop) << ";\n";
     o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(st.rop) << "; };\n";
-    for (int j = 0; j < NV; j++)
+    for (int j = 0; j < NV; j++) {
+      const bool guard = s.ragged && j == NV - 1;
+      if (guard) o << "  if (last_ok) {\n";
       for (int e = 0; e < V; e++)
         o << "  acc" << k << " = fold" << k << "((float)wkf_pre" << k << "(" << call_args(j, e, k) << "a.c + " << pre_off[k] << "), acc"
           << k << ");\n";
+      if (guard) o << "  }\n";
+    }
     if (T > 1) o << "  acc" << k << " = wkf_lanes_fold_with<" << std::min(T, 64) << ">(acc" << k << ", fold" << k << ");\n";
     if (T > 64) {
       const int WPR = T / 64;
@@ -953,7 +961,8 @@ std::string row_source(const RowSpec& s) {
       if (V > 1) o << "[" << e << "]";
       o << " = wkf_final(" << call_args(j, e, S) << "a.c + " << final_off << ");\n";
     }
-    o << "    __builtin_nontemporal_store(o" << j << ", (" << vt << "*)(qo + (t + " << j * T << "u) * " << V << "u));\n";
+    o << "    " << (s.ragged && j == NV - 1 ? "if (last_ok) " : "") << "__builtin_nontemporal_store(o" << j << ", (" << vt << "*)(qo + (t + " << j * T
+      << "u) * " << V << "u));\n";
   }
   o << "  }\n}\n";
   return o.str();
@@ -967,6 +976,7 @@ std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a) {
   std::vector<unsigned char> b;
   for (void* p : a.ptrs) putp(b, p);
   put32(b, a.nrows);
+  if (s.ragged) put32(b, a.nvec);
   for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? a.oshape[d] : 1);
   for (uint32_t v : a.offsets) put32(b, v);
   for (const auto& st : a.ostrides) {

@@ -137,7 +137,10 @@ struct RowSpec {
   int vec;                              // elements per 16-byte load
   int threads_per_row;                  // T
   int block;                            // threads per block
-  int vectors_per_lane;                 // NV: row length = NV * T * vec exactly
+  int vectors_per_lane;                 // NV: row length = NV * T * vec exactly, unless `ragged`
+  // ragged: the row holds `nvec` vectors (a launch argument) with (NV - 1) * T < nvec <= NV * T; lanes whose last
+  // vector lies past the end of the row neither load, fold nor store it
+  bool ragged = false;
   std::vector<ReduceOperandSpec> in;    // axis_stride 1 (row in registers) or 0 (one scalar per row)
   std::vector<RowStage> stages;
   Program final;                        // same operand numbering as a stage's pre
@@ -152,6 +155,7 @@ std::string row_source(const RowSpec& s);
 struct RowArgs {
   std::vector<void*> ptrs;                        // inputs..., out (store_scalars: one out per stage)
   uint32_t nrows;
+  uint32_t nvec = 0;                              // ragged kernels only: vectors per row
   std::vector<uint32_t> oshape;
   std::vector<uint32_t> offsets;                  // per operand incl. outputs
   std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. outputs, per outer dim

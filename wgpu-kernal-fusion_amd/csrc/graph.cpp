@@ -605,8 +605,8 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   RowSpec spec;
   size_t max_elem = scalars ? 2 : dtype_size(final.result_dtype());
   for (const TensorData& td : rb.operands) max_elem = std::max(max_elem, dtype_size(td.dtype));
-  const int V = int(16 / max_elem);
-  if (n == 0 || n % V) return false;
+  const int Vmax = int(16 / max_elem);
+  if (n == 0) return false;
   std::vector<size_t> out_shape(rb.shape.begin(), rb.shape.end() - 1);
   std::vector<std::vector<size_t>> ostr;
   for (const TensorData& td : rb.operands) ostr.push_back(std::vector<size_t>(td.layout.strides.begin(), td.layout.strides.end() - 1));
@@ -619,27 +619,47 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   if (Ro > 3) return false;
   for (size_t k = 0; k < K; k++) {
     const TensorData& td = rb.operands[k];
-    const size_t as = td.layout.strides[axis];
-    if (as > 1) return false;
-    if (as == 1) {
-      if (td.layout.offset % V) return false;
-      for (size_t d = 0; d < Ro; d++)
-        if (sp.strides[k][d] % V) return false;
-    }
+    if (td.layout.strides[axis] > 1) return false;
     if (td.layout.extent() > 0xffffffffull) return false;
-    spec.in.push_back({td.dtype, int(as)});
+    spec.in.push_back({td.dtype, int(td.layout.strides[axis])});
   }
+  // The widest vector (16 bytes down to one element) that divides the row and on which every row of every
+  // operand, and of the output when it has full rows, starts aligned
+  auto aligned = [&](int v) {
+    if (n % size_t(v)) return false;
+    for (size_t k = 0; k < K + (scalars ? 0 : NOUT); k++) {
+      if (k < K && rb.operands[k].layout.strides[axis] != 1) continue;
+      if (k < K && rb.operands[k].layout.offset % size_t(v)) return false;
+      for (size_t d = 0; d < Ro; d++)
+        if (sp.strides[k][d] % size_t(v)) return false;
+    }
+    return true;
+  };
+  int V = Vmax;
+  while (V > 1 && !aligned(V)) V /= 2;
   const size_t nvec = n / V;
+  // a lane holds at most 16 vectors of each operand; narrower vectors may be more (the same registers), for
+  // rows that no number of lanes covers otherwise
+  const size_t max_nv = size_t(16 * (Vmax / V));
   // Lanes per row, measured on MI355X: two 16-byte vectors per lane up to 256 lanes (softmax over 2048
   // floats: 169 us with 256 lanes, 173 with 64; RMSNorm over 4096: 15.9 us with 256, 17.2 with 128), more
   // lanes only when a lane would otherwise hold more than 16 vectors.
-  int T = std::min(256, pow2_ceil((nvec + 1) / 2));
-  while (T < 1024 && nvec > size_t(T) * 16) T *= 2;
-  while (T > 1 && nvec % size_t(T)) T /= 2;  // the row must split evenly over the lanes
+  const int T_wide = [&] {
+    int t = std::min(256, pow2_ceil((nvec + 1) / 2));
+    while (t < 1024 && nvec > size_t(t) * 16) t *= 2;
+    return t;
+  }();
+  int T = T_wide;
+  while (T > 1 && nvec % size_t(T)) T /= 2;  // first choice: the row splits evenly over the lanes
   if (st_.row_threads > 0 && size_t(st_.row_threads) <= nvec) T = st_.row_threads;
-  if (nvec % T) return false;
-  const size_t NV = nvec / T;
-  if (NV > 16 || NV * V * K > 128) return false;
+  bool ragged = false;
+  if (nvec % T || nvec / T > 16 || (nvec / T) * V * K > 128) {
+    // otherwise the widest layout, with the lanes past the end of the row masked in their last vector
+    T = T_wide;
+    ragged = true;
+  }
+  const size_t NV = (nvec + T - 1) / T;
+  if (NV > max_nv || NV * V * K > 128) return false;
   size_t nrows = 1;
   for (size_t d : out_shape) nrows *= d;
   if (nrows > 0xffffffffull) return false;
@@ -656,6 +676,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   spec.threads_per_row = T;
   spec.block = std::max(256, T);
   spec.vectors_per_lane = int(NV);
+  spec.ragged = ragged;
   spec.stages = rb.stages;
   spec.final = final;
   spec.store_scalars = scalars;
@@ -669,6 +690,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
 
   RowArgs args;
   args.nrows = uint32_t(nrows);
+  args.nvec = uint32_t(nvec);
   for (size_t d = 0; d < Ro; d++) args.oshape.push_back(to_u32(sp.shape[d], "shape"));
   for (size_t k = 0; k < K + NOUT; k++) {
     const TensorData& td = k < K ? rb.operands[k] : (*outs)[k - K];
@@ -696,6 +718,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   d << "rows=" << nrows << " n=" << n << " vec=" << V << " threads_per_row=" << T << " vectors_per_lane=" << NV << " stages="
     << rb.stages.size() << " operands=" << K + NOUT;
   if (scalars) d << " reductions=" << S;
+  if (ragged) d << " ragged";
   r.detail = d.str();
   record(std::move(r), k, row_pack_args(spec, args));
   return true;
