@@ -404,6 +404,14 @@ def test_row_kernel_takes_rows_that_do_not_split_evenly(wkf, planner):
     assert _kinds(long_rows) == ["red_row", "red_row", "map"]
 
 
+def test_f16_column_max_with_a_post_op_compiles(wkf, planner):
+    # this kernel (8 f16 columns per lane, 16 waves, four loads in flight, c - max) once hit a fatal "cannot select"
+    # error inside the compiler's backend, which ends the process; kernels are compiled without the SLP vectoriser since
+    t = 1.0 - _x(wkf, planner, (512, 8), np.float16).max(0)
+    assert _kinds(t) == ["red_col"] and t.shape() == (8,)
+    assert "|v8|" in t.kernels()[0].signature and "const_subtract" in t.kernels()[0].signature
+
+
 def test_mat_mul_kernel_choice(wkf, planner):
     def detail(m, n, k, dtype):
         t = _x(wkf, planner, (m, k), dtype).mat_mul(_x(wkf, planner, (k, n), dtype, seed=1))

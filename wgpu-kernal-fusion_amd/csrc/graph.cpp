@@ -2,6 +2,8 @@
 
 #include <algorithm>
 #include <functional>
+#include <cstdio>
+#include <cstdlib>
 #include <mutex>
 #include <set>
 #include <unordered_map>
@@ -256,6 +258,13 @@ wkf_kernel* Resolver::kernel(const std::string& sig, const std::function<std::st
   {
     std::lock_guard<std::mutex> lock(g_source_mu);
     g_sources.emplace(sig, src);
+  }
+  if (const char* dir = getenv("WKF_DUMP_SOURCES")) {
+    // every kernel's text as it goes to the compiler, "<dir>/<entry>.hip" (signature in the first line)
+    if (FILE* f = fopen((std::string(dir) + "/" + entry + ".hip").c_str(), "w")) {
+      fprintf(f, "// %s\n%s", sig.c_str(), src.c_str());
+      fclose(f);
+    }
   }
   wkf_kernel* k = nullptr;
   check(wkf_module_get(dev_, sig.c_str(), src.c_str(), entry.c_str(), &k));

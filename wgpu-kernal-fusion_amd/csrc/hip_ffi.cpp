@@ -40,8 +40,12 @@ int fail(int code, const std::string& msg) {
 
 // Options every kernel is compiled with.  -ffp-contract=off keeps each fused op
 // rounded on its own (no cross-op FMA); packed-fp32 code generation is disabled.
+// -fno-slp-vectorize: with packed fp32 off, the SLP vectorizer still forms <2 x float>
+// operations that the backend then cannot select ("Cannot select: v2f32 = bitcast", a fatal
+// compiler error that takes the process down; seen on an f16 column max).  The kernels
+// carry their own vector loads and stores, so nothing is lost.
 const char* const kCompileOptions[] = {
-    "--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-std=c++17",
+    "--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-std=c++17", "-fno-slp-vectorize",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 };
 constexpr int kNumCompileOptions = sizeof(kCompileOptions) / sizeof(kCompileOptions[0]);
