@@ -460,6 +460,15 @@ def test_batched_mat_mul_is_one_launch(wkf, planner):
     assert out.kernels()[2].detail.endswith("edge batch=8")    # n = 128 is half a tile: the edge kernel
     r4 = _x(wkf, planner, (2, 3, 17, 33), np.float32).mat_mul(_x(wkf, planner, (2, 3, 33, 5), np.float32, seed=1))
     assert r4.shape() == (2, 3, 17, 5) and _kinds(r4) == ["gemm"] and r4.kernels()[0].detail.endswith("generic batch=6")
+    # decode: one query row per head streams k and v once (the bandwidth kernels), one fold for all heads
+    q1 = _x(wkf, planner, (8, 1, 128), np.float16, seed=3)
+    kv = _x(wkf, planner, (8, 2048, 128), np.float16, seed=4)
+    s1 = q1.mat_mul(kv.transpose(1, 2))
+    assert _kinds(s1)[0] == "gemm" and len(_kinds(s1)) == 2           # the product, then the fold over the K slices
+    assert "skinny B^T" in s1.kernels()[0].detail and s1.kernels()[0].detail.endswith("batch=8")
+    o1 = s1.mat_mul(kv)
+    assert o1.shape() == (8, 1, 128) and _kinds(o1)[-2:] == ["gemm", "red_col"]
+    assert "skinny slices" in o1.kernels()[-2].detail and o1.kernels()[-2].detail.endswith("batch=8")
     # the same binaries as a single product: no new module for the batch
     before = planner.module_stats()
     _x(wkf, planner, (3, 256, 64), np.float16).mat_mul(_x(wkf, planner, (3, 64, 256), np.float16, seed=1)).materialize()

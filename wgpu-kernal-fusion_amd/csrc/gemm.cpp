@@ -96,7 +96,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   }
   const size_t V = a.dtype == DType::F16 ? 8 : 4;
   // ... and with up to 32 rows of A (decode) W is streamed once, straight into MFMA operands
-  const bool skinny_bt = batch == 1 && b_is_t && M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);
+  const bool skinny_bt = b_is_t && M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);
   bool bt = false;
   if (skinny_bt) {
     // handled below
@@ -108,8 +108,13 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (M == 0 || N == 0 || batch == 0) return alloc(out_shape, a.dtype, false);
   if (batch > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: more than 65535 matrices in a batch");
   if (M > 0xffffffffull || N > 0xffffffffull || K > 0xffffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: dimension does not fit 32 bits");
+  auto slices_shape = [&](size_t slices) {  // partial sums: [slice][batch...][M][N]
+    std::vector<size_t> sh = {slices};
+    sh.insert(sh.end(), out_shape.begin(), out_shape.end());
+    return sh;
+  };
   auto fold_slices = [&](const TensorData& part) {
-    // adds the f32 partial sums of the K slices ([S][M][N]) and rounds to the tensor dtype
+    // adds the f32 partial sums of the K slices ([S][batch...][M][N]) and rounds to the tensor dtype
     ReduceJob fold;
     Instr ld;
     ld.op = Op::Load;
@@ -129,14 +134,14 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (skinny_bt) {
     const size_t kblock = 128 / dtype_size(a.dtype);  // 128 bytes of every row per step
     const size_t gridx = (N + 127) / 128;
-    size_t S = (2048 + gridx - 1) / gridx;
+    size_t S = (2048 + gridx * batch - 1) / (gridx * batch);
     S = std::min(S, std::max<size_t>(1, K * dtype_size(a.dtype) / (8 * M)));  // partial sums stay under half of W's bytes
     S = std::min(S, std::max<size_t>(1, K / (2 * kblock)));
     size_t chunk = (K + S - 1) / S;
     chunk = (chunk + kblock - 1) / kblock * kblock;
     S = (K + chunk - 1) / chunk;
     if (S > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many K slices");
-    TensorData part = alloc({S, M, N}, DType::F32, false);
+    TensorData part = alloc(slices_shape(S), DType::F32, false);
     const std::string sig = std::string("gemm|gfx950|") + dtype_name(a.dtype) + "|skinny_bt|mfma32x32";
     wkf_kernel* k = kernel(sig, [&] { return std::string("#define WKF_H ") + (a.dtype == DType::F16 ? "1" : "0") + "\n" + kGemmSkinnyBt; });
     struct {
@@ -154,18 +159,20 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.block[0] = 256;
     r.grid[0] = uint32_t(gridx);
     r.grid[1] = uint32_t(S);
+    r.grid[2] = uint32_t(batch);
     std::ostringstream d;
     d << "m=" << M << " n=" << N << " k=" << K << " skinny B^T slices=" << S;
+    if (batch > 1) d << " batch=" << batch;
     r.detail = d.str();
     record(std::move(r), k, sbytes);
     return fold_slices(part);
   }
   // A handful of rows (decode): reading B once is all the work -> the bandwidth kernel, K cut into slices
   // across the grid, then one reduce launch that adds the slices and rounds to the tensor dtype.
-  if (st_.fusion == FusionMode::Tree && batch == 1 && !bt && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
+  if (st_.fusion == FusionMode::Tree && !bt && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
     const size_t esize = dtype_size(a.dtype);
     const size_t colblocks = (N + 256 * V - 1) / (256 * V);
-    size_t S = (1024 + colblocks - 1) / colblocks;
+    size_t S = (1024 + colblocks * batch - 1) / (colblocks * batch);
     S = std::min(S, std::max<size_t>(1, K * esize / (8 * M)));  // partial sums stay under half of B's bytes
     S = std::min(S, K / 16);
     S = std::max<size_t>(S, 1);
@@ -173,7 +180,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     chunk = (chunk + 3) & ~size_t(3);
     S = (K + chunk - 1) / chunk;
     if (S > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many K slices");
-    TensorData part = alloc({S, M, N}, DType::F32, false);
+    TensorData part = alloc(slices_shape(S), DType::F32, false);
     std::ostringstream sg;
     sg << "gemm|gfx950|" << dtype_name(a.dtype) << "|skinny|m" << M << "|v" << V;
     const std::string sig = sg.str();
@@ -198,8 +205,10 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.block[0] = 256;
     r.grid[0] = uint32_t(colblocks);
     r.grid[1] = uint32_t(S);
+    r.grid[2] = uint32_t(batch);
     std::ostringstream d;
     d << "m=" << M << " n=" << N << " k=" << K << " skinny slices=" << S;
+    if (batch > 1) d << " batch=" << batch;
     r.detail = d.str();
     record(std::move(r), k, sbytes);
 
