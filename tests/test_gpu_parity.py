@@ -616,7 +616,9 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                # a handful of rows (decode): the bandwidth kernel, K cut into slices, then a reduce over the slices
                # few tiles over a long K: K is cut into slices across the grid (f32 partial sums + a reduce)
                (300, 264, 2048), (128, 1032, 4096), (512, 512, 8192), (256, 256, 2048), (40, 512, 1096),
-               (1, 1024, 512), (5, 2048, 300), (16, 520, 1000), (8, 264, 4096), (2, 96, 8192), (3, 4104, 77)]
+               (1, 1024, 512), (5, 2048, 300), (16, 520, 1000), (8, 264, 4096), (2, 96, 8192), (3, 4104, 77),
+               # rows of B off the 16-byte grid (N odd): a transposed copy of B keeps a large product on the MFMA kernels
+               (300, 1001, 512), (512, 1002, 256), (17, 1003, 4096), (1, 5001, 4096)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -654,7 +656,8 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 ((8,), 512, 512, 128, True), ((8,), 512, 128, 512, False), ((2, 2), 300, 264, 72, True), ((6,), 1, 384, 128, True),
                 ((3,), 20, 100, 64, True), ((1,), 256, 512, 128, False), ((70,), 64, 64, 32, False),
                 # decode-sized products per matrix: the bandwidth kernels, K in slices, one fold for the batch
-                ((32,), 1, 2048, 128, True), ((32,), 1, 128, 2048, False), ((4,), 8, 520, 1000, False), ((3, 2), 20, 264, 4096, True)]
+                ((32,), 1, 2048, 128, True), ((32,), 1, 128, 2048, False), ((4,), 8, 520, 1000, False), ((3, 2), 20, 264, 4096, True),
+                ((3,), 300, 1001, 128, False)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

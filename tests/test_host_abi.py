@@ -426,6 +426,9 @@ def test_mat_mul_kernel_choice(wkf, planner):
     # unaligned rows or tiny problems: the generic kernel
     assert detail(300, 262, 72, np.float16).endswith("generic")
     assert detail(3, 7, 5, np.float32).endswith("generic")
+    # ... unless the product is large: then one transposed copy of B (rows aligned again) keeps it on the MFMA kernels
+    t = _x(wkf, planner, (300, 512), np.float16).mat_mul(_x(wkf, planner, (512, 1001), np.float16, seed=1))
+    assert _kinds(t) == ["map", "gemm"] and "tiled" in t.kernels()[0].detail and t.kernels()[1].detail.endswith("edge B^T")
     # a handful of rows: the bandwidth kernel over slices of K, then one reduce over the slices
     s = _x(wkf, planner, (4, 4096), np.float16).mat_mul(_x(wkf, planner, (4096, 2048), np.float16, seed=1))
     assert _kinds(s) == ["gemm", "red_col"] and "skinny" in s.kernels()[0].detail and s.shape() == (4, 2048)

@@ -95,8 +95,21 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     b_is_t = w.is_contiguous();
   }
   const size_t V = a.dtype == DType::F16 ? 8 : 4;
+  const bool decode_bt = M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);  // what the M <= 32 kernel for B^T takes
+  if (!b_is_t && st_.fusion == FusionMode::Tree && N % V != 0 && M * N * K >= (size_t(1) << 24) &&
+      (decode_bt || gemm_pick(a.dtype, M, N, K, true) != GemmKind::Generic)) {
+    // Rows of B that do not start on 16 bytes (N odd, say) would leave a large product to the generic kernel:
+    // a transposed copy of B (k contiguous, rows aligned because K is) costs one pass over B and keeps it on MFMA.
+    TensorData view = b;
+    std::swap(view.layout.shape[R - 2], view.layout.shape[R - 1]);
+    std::swap(view.layout.strides[R - 2], view.layout.strides[R - 1]);
+    b = make_contiguous(view);  // dense [..., N, K]
+    std::swap(b.layout.shape[R - 2], b.layout.shape[R - 1]);
+    std::swap(b.layout.strides[R - 2], b.layout.strides[R - 1]);  // seen as [..., K, N] again: the transpose of a dense matrix
+    b_is_t = true;
+  }
   // ... and with up to 32 rows of A (decode) W is streamed once, straight into MFMA operands
-  const bool skinny_bt = b_is_t && M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);
+  const bool skinny_bt = b_is_t && decode_bt;
   bool bt = false;
   if (skinny_bt) {
     // handled below
