@@ -29,7 +29,8 @@ constexpr size_t kSkinnyRows = 16;  // most rows of A the bandwidth kernel takes
 GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k, bool b_transposed) {
   if (m == 0 || n == 0 || k == 0) return GemmKind::Generic;
   const bool whole = m % 256 == 0 && n % 256 == 0;
-  if (dt == DType::F16 && whole && k % 64 == 0) return GemmKind::MfmaF16;
+  // (the full-tile f16 kernel addresses a tile's rows with 32-bit byte offsets from the tile origin)
+  if (dt == DType::F16 && whole && k % 64 == 0 && k <= (size_t(1) << 21) && n <= (size_t(1) << 22)) return GemmKind::MfmaF16;
   if (dt == DType::F32 && whole && k % 32 == 0) return GemmKind::MfmaF32;
   // ragged shapes keep the MFMA kernels as long as every row of A and B starts on a 16-byte boundary
   // and the problem is worth a 256 x 256 tile; tiny or unaligned ones take the generic kernel
