@@ -618,7 +618,9 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                (300, 264, 2048), (128, 1032, 4096), (512, 512, 8192), (256, 256, 2048), (40, 512, 1096),
                (1, 1024, 512), (5, 2048, 300), (16, 520, 1000), (8, 264, 4096), (2, 96, 8192), (3, 4104, 77),
                # rows of B off the 16-byte grid (N odd): a transposed copy of B keeps a large product on the MFMA kernels
-               (300, 1001, 512), (512, 1002, 256), (17, 1003, 4096), (1, 5001, 4096)]
+               (300, 1001, 512), (512, 1002, 256), (17, 1003, 4096), (1, 5001, 4096),
+               # K off the vector grid: zero-padded copies of A and B keep a large product on the MFMA kernels
+               (300, 1000, 515), (512, 512, 1001), (300, 1001, 515)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -634,7 +636,7 @@ def test_mat_mul(gpu, m, n, k, dtype, tol):
 
 
 BT_SHAPES = [(256, 512, 128), (300, 264, 2048), (100, 136, 72), (513, 260, 328), (1, 1024, 512), (7, 520, 1000),
-             (32, 264, 4096), (2, 4100, 96), (20, 100, 64), (3, 5, 7), (33, 2048, 1024)]
+             (32, 264, 4096), (2, 4100, 96), (20, 100, 64), (3, 5, 7), (33, 2048, 1024), (300, 1000, 515)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

@@ -429,6 +429,9 @@ def test_mat_mul_kernel_choice(wkf, planner):
     # ... unless the product is large: then one transposed copy of B (rows aligned again) keeps it on the MFMA kernels
     t = _x(wkf, planner, (300, 512), np.float16).mat_mul(_x(wkf, planner, (512, 1001), np.float16, seed=1))
     assert _kinds(t) == ["map", "gemm"] and "tiled" in t.kernels()[0].detail and t.kernels()[1].detail.endswith("edge B^T")
+    # ... and when K is off the vector grid, zero-padded copies of both operands do
+    t = _x(wkf, planner, (300, 515), np.float16).mat_mul(_x(wkf, planner, (515, 1000), np.float16, seed=1))
+    assert _kinds(t) == ["map", "map", "gemm"] and "k=520" in t.kernels()[2].detail and t.shape() == (300, 1000)
     # a handful of rows: the bandwidth kernel over slices of K, then one reduce over the slices
     s = _x(wkf, planner, (4, 4096), np.float16).mat_mul(_x(wkf, planner, (4096, 2048), np.float16, seed=1))
     assert _kinds(s) == ["gemm", "red_col"] and "skinny" in s.kernels()[0].detail and s.shape() == (4, 2048)

@@ -78,7 +78,8 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     batch *= a.layout.shape[d];
     out_shape.push_back(a.layout.shape[d]);
   }
-  const size_t M = a.layout.shape[R - 2], K = a.layout.shape[R - 1], N = b.layout.shape[R - 1];
+  const size_t M = a.layout.shape[R - 2], N = b.layout.shape[R - 1];
+  size_t K = a.layout.shape[R - 1];
   if (b.layout.shape[R - 2] != K) invalid("mat_mul: inner dimensions differ");  // src/matmul.rs:194
   out_shape.push_back(M);
   out_shape.push_back(N);
@@ -96,6 +97,41 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     b_is_t = w.is_contiguous();
   }
   const size_t V = a.dtype == DType::F16 ? 8 : 4;
+  if (st_.fusion == FusionMode::Tree && K % V != 0 && M * N * K >= (size_t(1) << 24)) {
+    // Rows of A (and of a transposed B) that do not start on 16 bytes because K is odd, say: zero-padded copies up to
+    // the next multiple of the vector keep a large product on the MFMA kernels; the zeros add nothing to the sums.
+    const size_t Kp = (K + V - 1) / V * V;
+    auto pad_dim = [&](const TensorData& t, size_t dim) {  // t dense; returns a dense copy with `dim` grown to Kp
+      std::vector<size_t> shape = t.layout.shape;
+      shape[dim] = Kp;
+      TensorData out = alloc(shape, t.dtype, true);
+      std::vector<std::pair<size_t, size_t>> corner;
+      for (size_t d = 0; d < shape.size(); d++) corner.push_back({0, t.layout.shape[d]});
+      TensorData view = out;
+      view.layout = out.layout.slice(corner);
+      Program p;
+      Instr in;
+      in.op = Op::Load;
+      in.dtype = t.dtype;
+      in.operand = 0;
+      p.ins.push_back(in);
+      p.result = 0;
+      launch_map(p, {t}, view, false);
+      return out;
+    };
+    a = pad_dim(a, R - 1);
+    if (b_is_t) {
+      TensorData w = b;  // the dense [..., N, K] behind the transposed view
+      std::swap(w.layout.shape[R - 2], w.layout.shape[R - 1]);
+      std::swap(w.layout.strides[R - 2], w.layout.strides[R - 1]);
+      b = pad_dim(w, R - 1);
+      std::swap(b.layout.shape[R - 2], b.layout.shape[R - 1]);
+      std::swap(b.layout.strides[R - 2], b.layout.strides[R - 1]);
+    } else {
+      b = pad_dim(make_contiguous(b), R - 2);
+    }
+    K = Kp;
+  }
   const bool decode_bt = M >= 1 && M <= 32 && K % V == 0 && N * K >= (size_t(1) << 16);  // what the M <= 32 kernel for B^T takes
   if (!b_is_t && st_.fusion == FusionMode::Tree && N % V != 0 && M * N * K >= (size_t(1) << 24) &&
       (decode_bt || gemm_pick(a.dtype, M, N, K, true) != GemmKind::Generic)) {
