@@ -184,7 +184,10 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (skinny_bt) {
     const size_t kblock = 128 / dtype_size(a.dtype);  // 128 bytes of every row per step
     const size_t gridx = (N + 127) / 128;
-    size_t S = (2048 + gridx * batch - 1) / (gridx * batch);
+    // workgroups to aim for, from a sweep on MI355X ([M x 4096] x W[11008 x 4096]^T and W[4096 x 4096]^T): more slices
+    // fill the chip, fewer keep the f32 partial sums (written and read once more by the fold) small as M grows
+    const size_t want = st_.skinny_blocks > 0 ? size_t(st_.skinny_blocks) : (M >= 16 ? 512 : 1024);
+    size_t S = (want + gridx * batch - 1) / (gridx * batch);
     S = std::min(S, std::max<size_t>(1, K * dtype_size(a.dtype) / (8 * M)));  // partial sums stay under half of W's bytes
     S = std::min(S, std::max<size_t>(1, K / (2 * kblock)));
     size_t chunk = (K + S - 1) / S;
@@ -222,7 +225,8 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (st_.fusion == FusionMode::Tree && !bt && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
     const size_t esize = dtype_size(a.dtype);
     const size_t colblocks = (N + 256 * V - 1) / (256 * V);
-    size_t S = (1024 + colblocks * batch - 1) / (colblocks * batch);
+    const size_t want = st_.skinny_blocks > 0 ? size_t(st_.skinny_blocks) : 1024;
+    size_t S = (want + colblocks * batch - 1) / (colblocks * batch);
     S = std::min(S, std::max<size_t>(1, K * esize / (8 * M)));  // partial sums stay under half of B's bytes
     S = std::min(S, K / 16);
     S = std::max<size_t>(S, 1);
