@@ -26,7 +26,9 @@ const char* const kGemmSkinnyBt =
 const char* const kGemmSkinnyTr =
 #include "kernels/gemm_skinny_tr.hip.inc"
     ;
-constexpr size_t kSkinnyRows = 16;  // most rows of A the bandwidth kernel takes (accumulators: rows x 8 per lane)
+// most rows of A the lane-per-column bandwidth kernel takes (accumulators: rows x 8 per lane for f16, rows x 4 for f32;
+// f32 has no MFMA decode kernel for a row-major B, and a 256-row MFMA tile for 32 rows of f32 is 3 times slower still)
+constexpr size_t kSkinnyRowsF16 = 16, kSkinnyRowsF32 = 32;
 }  // namespace
 
 GemmKind gemm_pick(DType dt, size_t m, size_t n, size_t k, bool b_transposed) {
@@ -268,7 +270,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   }
   // A handful of rows (decode): reading B once is all the work -> the bandwidth kernel, K cut into slices
   // across the grid, then one reduce launch that adds the slices and rounds to the tensor dtype.
-  if (st_.fusion == FusionMode::Tree && !bt && M <= kSkinnyRows && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
+  if (st_.fusion == FusionMode::Tree && !bt && M <= (a.dtype == DType::F16 ? kSkinnyRowsF16 : kSkinnyRowsF32) && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
     const size_t esize = dtype_size(a.dtype);
     const size_t colblocks = (N + 256 * V - 1) / (256 * V);
     const size_t want = st_.skinny_blocks > 0 ? size_t(st_.skinny_blocks) : 1024;
