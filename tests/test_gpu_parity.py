@@ -622,7 +622,9 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                # K off the vector grid: zero-padded copies of A and B keep a large product on the MFMA kernels
                (300, 1000, 515), (512, 512, 1001), (300, 1001, 515),
                # 5 to 32 rows against a row-major B: the MFMA decode kernel (LDS transpose reads), K in slices
-               (32, 4096, 512), (17, 264, 1000), (8, 1000, 4096), (31, 72, 2048), (5, 4104, 136), (24, 8, 8200), (32, 1028, 700)]
+               (32, 4096, 512), (17, 264, 1000), (8, 1000, 4096), (31, 72, 2048), (5, 4104, 136), (24, 8, 8200), (32, 1028, 700),
+               # 128 x 128 tiles (products that would not fill the chip with 256 x 256 ones): full, ragged, K in slices
+               (128, 128, 64), (129, 136, 64), (384, 640, 192), (200, 1000, 520), (511, 136, 2048), (33, 4096, 1024)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

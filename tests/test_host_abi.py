@@ -418,17 +418,21 @@ def test_mat_mul_kernel_choice(wkf, planner):
         assert _kinds(t) == ["gemm"]
         return t.kernels()[0].detail
 
-    assert detail(512, 256, 128, np.float16).endswith("mfma 256x256 tiles")
+    assert detail(4096, 4096, 128, np.float16).endswith("mfma 256x256 tiles")
     assert detail(512, 256, 96, np.float32).endswith("mfma 256x256 tiles")
     # not a multiple of the tile but every row 16-byte aligned: the same MFMA kernel with edge handling
-    assert detail(300, 264, 72, np.float16).endswith("mfma 256x256 tiles edge")
+    assert detail(4000, 4104, 72, np.float16).endswith("mfma 256x256 tiles edge")
     assert detail(300, 260, 68, np.float32).endswith("mfma 256x256 tiles edge")
+    # f16 products whose large tiles would fill at most half of the chip take 128 x 128 tiles, two workgroups per compute unit
+    assert detail(512, 256, 128, np.float16).endswith("mfma 128x128 tiles")
+    assert detail(300, 264, 72, np.float16).endswith("mfma 128x128 tiles")
+    assert detail(1024, 11008, 512, np.float16).endswith("mfma 256x256 tiles")
     # unaligned rows or tiny problems: the generic kernel
     assert detail(300, 262, 72, np.float16).endswith("generic")
     assert detail(3, 7, 5, np.float32).endswith("generic")
     # ... unless the product is large: then one transposed copy of B (rows aligned again) keeps it on the MFMA kernels
     t = _x(wkf, planner, (300, 512), np.float16).mat_mul(_x(wkf, planner, (512, 1001), np.float16, seed=1))
-    assert _kinds(t) == ["map", "gemm"] and "tiled" in t.kernels()[0].detail and t.kernels()[1].detail.endswith("edge B^T")
+    assert _kinds(t) == ["map", "gemm"] and "tiled" in t.kernels()[0].detail and t.kernels()[1].detail.endswith("tiles B^T")
     # ... and when K is off the vector grid, zero-padded copies of both operands do
     t = _x(wkf, planner, (300, 515), np.float16).mat_mul(_x(wkf, planner, (515, 1000), np.float16, seed=1))
     assert _kinds(t) == ["map", "map", "gemm"] and "k=520" in t.kernels()[2].detail and t.shape() == (300, 1000)
@@ -463,7 +467,7 @@ def test_batched_mat_mul_is_one_launch(wkf, planner):
     v = _x(wkf, planner, (8, 512, 128), np.float16, seed=2)
     out = scores.softmax_last_dim().mat_mul(v)
     assert out.shape() == (8, 512, 128) and _kinds(out) == ["gemm", "row", "gemm"]
-    assert out.kernels()[2].detail.endswith("edge batch=8")    # n = 128 is half a tile: the edge kernel
+    assert out.kernels()[2].detail.endswith("128x128 tiles batch=8")    # n = 128: the small tile, nothing wasted
     r4 = _x(wkf, planner, (2, 3, 17, 33), np.float32).mat_mul(_x(wkf, planner, (2, 3, 33, 5), np.float32, seed=1))
     assert r4.shape() == (2, 3, 17, 5) and _kinds(r4) == ["gemm"] and r4.kernels()[0].detail.endswith("generic batch=6")
     # decode: one query row per head streams k and v once (the bandwidth kernels), one fold for all heads

@@ -26,6 +26,9 @@ const char* const kGemmSkinnyBt =
 const char* const kGemmSkinnyTr =
 #include "kernels/gemm_skinny_tr.hip.inc"
     ;
+const char* const kGemmF16T128 =
+#include "kernels/gemm_f16_t128.hip.inc"
+    ;
 // most rows of A the lane-per-column bandwidth kernel takes (accumulators: rows x 8 per lane for f16, rows x 4 for f32;
 // f32 has no MFMA decode kernel for a row-major B, and a 256-row MFMA tile for 32 rows of f32 is 3 times slower still)
 constexpr size_t kSkinnyRowsF16 = 16, kSkinnyRowsF32 = 32;
@@ -323,14 +326,24 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // (f32 partial sums per slice, then one reduce launch), as long as the partial sums stay below
   // the bytes of A and B.
   size_t slices = 1, kchunk = 0;
+  wkf_props props;
+  if (wkf_device_props(dev_, &props) != WKF_OK) throw Error(WKF_ERR_HIP, wkf_last_error());
+  const size_t cus = size_t(std::max(1, props.compute_units));
+  // f16 products whose 256 x 256 tiles would fill at most half of the chip take 128 x 128 tiles, two workgroups per
+  // compute unit ([512 x 4096] x [4096 x 11008]: 92 us against 109; with 172 of the large tiles, [1024 x ...], the large
+  // tile is the faster one again: 119 us against 159)
+  const size_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
+  // ... and so do products that would waste half of every large tile (128 columns of attention values, say)
+  const size_t pad256 = ((M + 255) / 256 * 256) * ((N + 255) / 256 * 256), pad128 = ((M + 127) / 128 * 128) * ((N + 127) / 128 * 128);
+  const bool t128 = mfma && a.dtype == DType::F16 && st_.fusion == FusionMode::Tree && st_.gemm_t128 &&
+                    (tiles256 * batch * 2 <= cus || pad128 * 20 <= pad256 * 11);
+  const size_t tile = t128 ? 128 : 256;
+  const size_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
+  const size_t slots = t128 ? 2 * cus : cus;  // workgroups the chip holds at once
   if (mfma && batch == 1 && st_.fusion == FusionMode::Tree) {
-    wkf_props props;
-    if (wkf_device_props(dev_, &props) != WKF_OK) throw Error(WKF_ERR_HIP, wkf_last_error());
-    const size_t cus = size_t(std::max(1, props.compute_units));
-    const size_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
     const size_t bk = a.dtype == DType::F16 ? 64 : 32;
-    if (tiles * 2 <= cus && K >= 1024) {
-      size_t S = std::min((cus + tiles - 1) / tiles, K / 512);
+    if (tiles * 2 <= slots && K >= 1024) {
+      size_t S = std::min((slots + tiles - 1) / tiles, K / 512);
       while (S > 1 && S * M * N * 4 > (M * K + K * N) * dtype_size(a.dtype)) S--;
       if (S > 1) {
         kchunk = (K + S - 1) / S;
@@ -341,11 +354,12 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   }
   const bool split = slices > 1;
   TensorData out = split ? alloc({slices, M, N}, DType::F32, false) : alloc(out_shape, a.dtype, false);
-  std::string sig = gemm_signature(kind, a.dtype);
+  std::string sig = t128 ? std::string("gemm|gfx950|f16|mfma32x32x16|128x128x64|w2x2|edge") : gemm_signature(kind, a.dtype);
   if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
   if (bt) sig += "|bt";
   wkf_kernel* k = kernel(sig, [&] {
     std::string src = bt ? "#define WKF_BT 1\n" : "";
+    if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + kGemmF16T128;
     if (!split) return src + gemm_source(kind, a.dtype);
     const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
     return src + "#define WKF_SPLITK 1\n" + gemm_source(base, a.dtype);
@@ -370,15 +384,14 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.grid[1] = uint32_t((M + 63) / 64);
     if (r.grid[1] > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many rows for the generic kernel");
   } else {
-    const size_t tiles = ((M + 255) / 256) * ((N + 255) / 256);
     if (tiles > 0x7fffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
     r.grid[0] = uint32_t(tiles);
     r.grid[1] = uint32_t(slices);
   }
   r.grid[2] = uint32_t(batch);
   std::ostringstream d;
-  d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : " mfma 256x256 tiles");
-  if (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge) d << " edge";
+  d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : t128 ? " mfma 128x128 tiles" : " mfma 256x256 tiles");
+  if (!t128 && (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge)) d << " edge";
   if (bt) d << " B^T";
   if (split) d << " slices=" << slices;
   if (batch > 1) d << " batch=" << batch;
