@@ -343,7 +343,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (mfma && batch == 1 && st_.fusion == FusionMode::Tree) {
     const size_t bk = a.dtype == DType::F16 ? 64 : 32;
     if (tiles * 2 <= slots && K >= 1024) {
-      size_t S = std::min((slots + tiles - 1) / tiles, K / 512);
+      size_t S = std::min(std::max<size_t>(1, slots / tiles), K / 512);  // rounded down: one workgroup more than the chip holds costs a second round
       while (S > 1 && S * M * N * 4 > (M * K + K * N) * dtype_size(a.dtype)) S--;
       if (S > 1) {
         kchunk = (K + S - 1) / S;
