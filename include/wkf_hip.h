@@ -53,6 +53,10 @@ int wkf_device_create(int ordinal, wkf_device** out);
  * fusion and code generation can be tested on a machine without a GPU; it
  * computes nothing.  No counterpart in the reference. */
 int wkf_device_create_planner(wkf_device** out);
+/* Drops the caller's handle.  While buffers of the device (or tensors that own some) are still alive the device
+ * itself lives on and is torn down by the release of the last one, so a late wkf_buffer_release /
+ * wkf_tensor_free is always safe; no new work may be started through the handle after this call.  Timers
+ * are not counted: destroy them first. */
 void wkf_device_destroy(wkf_device* dev);
 int wkf_device_is_planner(const wkf_device* dev);
 /* Replaces wgpu_device().limits(), src/reduce.rs:340. */

@@ -663,7 +663,11 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 ((3,), 20, 100, 64, True), ((1,), 256, 512, 128, False), ((70,), 64, 64, 32, False),
                 # decode-sized products per matrix: the bandwidth kernels, K in slices, one fold for the batch
                 ((32,), 1, 2048, 128, True), ((32,), 1, 128, 2048, False), ((4,), 8, 520, 1000, False), ((3, 2), 20, 264, 4096, True),
-                ((3,), 300, 1001, 128, False)]
+                ((3,), 300, 1001, 128, False),
+                # a batch of one with a long K: few tiles, so K is cut into slices (256 x 256 and 128 x 128 tiles); the
+                # leading dimensions of size 1 must survive the fold of the slices
+                ((1,), 256, 256, 4096, False), ((1, 1), 256, 512, 2048, True), ((1,), 128, 384, 4096, False),
+                ((1, 1), 100, 136, 1024, False)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -680,8 +684,11 @@ def test_batched_mat_mul(gpu, lead, m, n, k, bt, dtype, tol):
     dense_b = np.swapaxes(b, -1, -2) if bt else b
     first = tuple(0 for _ in lead)
     one = api.tensor(a[first]).mat_mul(api.tensor(np.ascontiguousarray(dense_b[first])))
-    got, alone = hip_values_many([prod, one])
+    # the product as an operand of a following pair-wise op: its recorded shape and its buffer's must agree
+    chained = prod + prod
+    got, alone, twice = hip_values_many([prod, one, chained])
     assert got.dtype == dtype and got.shape == lead + (m, n)
+    assert twice.shape == lead + (m, n) and np.array_equal(twice, got + got)
     for idx in np.ndindex(*lead):
         gemm_check(got[idx], a[idx], np.ascontiguousarray(dense_b[idx]), tol)
     assert len([kk for kk in prod.kernels() if kk.kind == "gemm"]) == 1

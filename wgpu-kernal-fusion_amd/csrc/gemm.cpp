@@ -353,7 +353,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     }
   }
   const bool split = slices > 1;
-  TensorData out = split ? alloc({slices, M, N}, DType::F32, false) : alloc(out_shape, a.dtype, false);
+  TensorData out = split ? alloc(slices_shape(slices), DType::F32, false) : alloc(out_shape, a.dtype, false);
   std::string sig = t128 ? std::string("gemm|gfx950|f16|mfma32x32x16|128x128x64|w2x2|edge") : gemm_signature(kind, a.dtype);
   if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
   if (bt) sig += "|bt";

@@ -1163,7 +1163,17 @@ TensorData Resolver::launch_reduce(const ReduceJob& job) {
   ostr.push_back(out.layout.strides);
   Space sp = coalesce(out_shape, ostr);
   const size_t Ro = sp.shape.size();
-  if (Ro > 3) throw Error(WKF_ERR_UNSUPPORTED, "reduce kernel: more than 3 non-mergeable outer dimensions");
+  if (Ro > 3) {
+    // The reduce kernels decode at most three outer dimensions (the reference's takes any rank, src/reduce.rs:83-281):
+    // a view whose outer dimensions do not merge that far is copied into a dense buffer first (one map pass, any
+    // rank up to the map kernel's), after which the dimensions on either side of the axis merge into one each.
+    bool dense = true;
+    for (const TensorData& td : ops) dense &= td.layout.is_contiguous();
+    if (dense) throw Error(WKF_ERR_UNSUPPORTED, "reduce kernel: more than 3 non-mergeable outer dimensions");
+    ReduceJob copy = job;
+    for (TensorData& td : copy.operands) td = make_contiguous(td);
+    return launch_reduce(copy);
+  }
 
   ReduceSpec spec;
   spec.outer_rank = int(Ro);

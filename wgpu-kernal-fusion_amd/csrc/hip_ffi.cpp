@@ -110,6 +110,12 @@ struct wkf_device {
   uint64_t n_compiled = 0, n_disk = 0, n_mem = 0;
   std::string cache_path;
   wkf_props props{};
+  // buffers handed out and not yet released; a destroy with some still alive is deferred to the last release
+  size_t live_buffers = 0;
+  bool closing = false;
+  // events of destroyed timers, handed out again by wkf_timer_create: a timed launch costs two event
+  // records, not two event creations and destructions
+  std::vector<hipEvent_t> free_events;
 };
 
 struct wkf_buffer {
@@ -219,8 +225,24 @@ int wkf_device_trim(wkf_device* dev) {
   return WKF_OK;
 }
 
+static void destroy_now(wkf_device* dev);
+
 void wkf_device_destroy(wkf_device* dev) {
   if (!dev) return;
+  {
+    // Buffers (and the tensors that own them) may outlive the caller's last use of the device handle: the device
+    // then lives on until the last of them is released, so that a late wkf_buffer_release / wkf_tensor_free
+    // never touches freed memory.
+    std::lock_guard<std::recursive_mutex> lock(dev->mu);
+    if (dev->live_buffers > 0) {
+      dev->closing = true;
+      return;
+    }
+  }
+  destroy_now(dev);
+}
+
+static void destroy_now(wkf_device* dev) {
   {
     std::vector<void (*)(wkf_device*)> hooks;
     {
@@ -234,6 +256,7 @@ void wkf_device_destroy(wkf_device* dev) {
     if (kv.second->module) hipModuleUnload(kv.second->module);
     delete kv.second;
   }
+  for (hipEvent_t e : dev->free_events) hipEventDestroy(e);
   if (dev->stream) hipStreamDestroy(dev->stream);
   delete dev;
 }
@@ -289,6 +312,7 @@ int wkf_buffer_alloc(wkf_device* dev, size_t bytes, int zero_fill, wkf_buffer** 
     }
   }
   wkf_buffer* b = new wkf_buffer{dev, ptr, bytes, cap, {1}, false};
+  dev->live_buffers++;
   *out = b;
   return WKF_OK;
 }
@@ -301,8 +325,10 @@ void wkf_buffer_release(wkf_buffer* buf) {
   if (!buf) return;
   if (buf->refs.fetch_sub(1, std::memory_order_acq_rel) != 1) return;
   wkf_device* dev = buf->dev;
+  bool last = false;
   {
     std::lock_guard<std::recursive_mutex> lock(dev->mu);
+    last = --dev->live_buffers == 0 && dev->closing;
     // Work already queued on the single stream finishes before any later user of
     // this block starts, so the block can be handed out again without a sync.
     if (dev->pool_bytes + buf->capacity <= dev->pool_limit) {
@@ -316,6 +342,7 @@ void wkf_buffer_release(wkf_buffer* buf) {
     }
   }
   delete buf;
+  if (last) destroy_now(dev);
 }
 
 int wkf_buffer_refcount(const wkf_buffer* buf) { return buf ? buf->refs.load(std::memory_order_acquire) : 0; }
@@ -519,10 +546,17 @@ int wkf_timer_create(wkf_device* dev, wkf_timer** out) {
   wkf_timer* t = new wkf_timer();
   t->dev = dev;
   if (!dev->planner) {
-    if (hipEventCreate(&t->begin) != hipSuccess || hipEventCreate(&t->end) != hipSuccess) {
-      if (t->begin) hipEventDestroy(t->begin);
-      delete t;
-      return fail(WKF_ERR_HIP, "hipEventCreate failed");
+    std::lock_guard<std::recursive_mutex> lock(dev->mu);
+    hipEvent_t* slot[2] = {&t->begin, &t->end};
+    for (hipEvent_t* e : slot) {
+      if (!dev->free_events.empty()) {
+        *e = dev->free_events.back();
+        dev->free_events.pop_back();
+      } else if (hipSetDevice(dev->ordinal) != hipSuccess || hipEventCreate(e) != hipSuccess) {
+        if (t->begin) dev->free_events.push_back(t->begin);
+        delete t;
+        return fail(WKF_ERR_HIP, "hipEventCreate failed");
+      }
     }
   }
   *out = t;
@@ -531,8 +565,11 @@ int wkf_timer_create(wkf_device* dev, wkf_timer** out) {
 
 void wkf_timer_destroy(wkf_timer* t) {
   if (!t) return;
-  if (t->begin) hipEventDestroy(t->begin);
-  if (t->end) hipEventDestroy(t->end);
+  {
+    std::lock_guard<std::recursive_mutex> lock(t->dev->mu);
+    if (t->begin) t->dev->free_events.push_back(t->begin);
+    if (t->end) t->dev->free_events.push_back(t->end);
+  }
   delete t;
 }
 
