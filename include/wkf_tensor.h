@@ -98,6 +98,18 @@ int wkf_tensor_cast(const wkf_tensor* t, int dtype, wkf_tensor** out);
 int wkf_tensor_binary_op(const wkf_tensor* a, const wkf_tensor* b, int op, wkf_tensor** out);
 /* Sum::sum / Max::max / Min::min / Product::product over `axis`; rank drops by one. */
 int wkf_tensor_reduce(const wkf_tensor* t, int reduce_op, size_t axis, wkf_tensor** out);
+/* wkf_tensor_reduce + wkf_tensor_materialize for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc); it has no counterpart in the reference.  `t` and
+ * `out` are dense tensors that hold data already (wkf_tensor_new), `out` with t's shape minus `axis` and t's dtype;
+ * the result is written into out's buffer with the same kernels, launches and bits as the allocating path.  The
+ * call allocates nothing on the device: no hipMalloc / hipFree, no code-object load, no event.  A reduction that is
+ * folded in two launches (few outputs over a long axis) keeps its f32 partial results in a file-scope device array
+ * of 1 MiB that every GPU the library runs on holds until the process ends; a reduction whose partial results need
+ * more is refused with WKF_ERR_INVALID_ARG.  The kernels must be loaded already: run the allocating path once on
+ * tensors of the same shape and dtype (else WKF_ERR_INVALID_ARG names the missing kernel).  Nothing in the array has
+ * to start at zero (the first launch overwrites every partial result the second reads), and it keeps the last
+ * call's contents.  All calls on one device share the array: calls that overlap on one device race. */
+int wkf_tensor_reduce_into(const wkf_tensor* t, int reduce_op, size_t axis, wkf_tensor* out);
 /* Tensor::mat_mul, src/matmul.rs:25-29: rank 2, same dtype, [M,K] x [K,N].  Beyond the reference (whose mat_mul
  * is rank 2 only): operands of equal rank > 2 are a batch, [..., M, K] x [..., K, N] -> [..., M, N] with equal
  * leading dimensions (at most 65535 matrices), one launch for all of them. */

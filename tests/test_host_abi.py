@@ -521,3 +521,31 @@ def test_generated_source_keeps_every_op_rounded_on_its_own(wkf, planner):
         assert "wkf_exp(v3)" in wkf.kernel_source(f.kernels()[0].signature)
     finally:
         planner.set_exact_math(False)
+
+
+def test_reduce_into_plans_without_allocating_and_refuses_the_rest(wkf):
+    # the allocation-free variant of reduce + materialize, on a device of its own (fresh kernel table)
+    dev = wkf.Device.planner()
+    T = wkf.Tensor
+    x = T.new(dev, np.zeros((64, 262144), dtype=np.float32))
+    out = T.new(dev, np.zeros((64,), dtype=np.float32))
+    # its kernels are not loaded yet: loading one would allocate, so the call names the kernel and stops
+    with pytest.raises(wkf.WkfError, match="is not loaded"):
+        x.reduce_into("sum", 1, out)
+    lazy = x.sum(1)
+    lazy.materialize()
+    assert len(lazy.kernels()) == 2  # few rows over a long axis: partial results, then the fold
+    before = dev.module_stats()
+    x.reduce_into("sum", 1, out)
+    after = dev.module_stats()
+    assert (after["compiled"], after["disk_hits"]) == (before["compiled"], before["disk_hits"])
+    # partial results beyond the static scratch array (1 MiB): refused with the sizes in the message
+    big = T.new(dev, np.zeros((4096, 32768), dtype=np.float16))
+    big.sum(0).materialize()
+    with pytest.raises(wkf.WkfError, match="static scratch array holds 1048576"):
+        big.reduce_into("sum", 0, T.new(dev, np.zeros((32768,), dtype=np.float16)))
+    with pytest.raises(wkf.WkfError, match="hold data"):
+        (x + 1.0).reduce_into("sum", 1, out)
+    with pytest.raises(wkf.WkfError, match="shape"):
+        x.reduce_into("sum", 1, T.new(dev, np.zeros((63,), dtype=np.float32)))
+    dev.close()

@@ -42,7 +42,7 @@ EXPORTS = [
     "wkf_last_error",
     "wkf_device_set_fusion", "wkf_device_get_fusion", "wkf_device_set_exact_math", "wkf_device_set_timing", "wkf_tensor_new", "wkf_tensor_clone", "wkf_tensor_free",
     "wkf_tensor_rank", "wkf_tensor_shape", "wkf_tensor_dtype", "wkf_tensor_scalar_op", "wkf_tensor_unary_op",
-    "wkf_tensor_cast", "wkf_tensor_binary_op", "wkf_tensor_reduce", "wkf_tensor_mat_mul", "wkf_tensor_slice",
+    "wkf_tensor_cast", "wkf_tensor_binary_op", "wkf_tensor_reduce", "wkf_tensor_reduce_into", "wkf_tensor_mat_mul", "wkf_tensor_slice",
     "wkf_tensor_transpose", "wkf_tensor_broadcast", "wkf_tensor_narrow", "wkf_tensor_resize",
     "wkf_tensor_reshape", "wkf_tensor_unsqueeze", "wkf_tensor_slice_assign", "wkf_tensor_cat", "wkf_tensor_silu",
     "wkf_tensor_layer_norm", "wkf_tensor_rope", "wkf_tensor_softmax", "wkf_tensor_softmax_last_dim",
@@ -93,6 +93,7 @@ def load():
     lib.wkf_tensor_cast.argtypes = [c_void_p, c_int, POINTER(c_void_p)]
     lib.wkf_tensor_binary_op.argtypes = [c_void_p, c_void_p, c_int, POINTER(c_void_p)]
     lib.wkf_tensor_reduce.argtypes = [c_void_p, c_int, c_size_t, POINTER(c_void_p)]
+    lib.wkf_tensor_reduce_into.argtypes = [c_void_p, c_int, c_size_t, c_void_p]
     lib.wkf_tensor_mat_mul.argtypes = [c_void_p, c_void_p, POINTER(c_void_p)]
     lib.wkf_tensor_new.argtypes = [c_void_p, c_int, c_int, POINTER(c_size_t), c_void_p, POINTER(c_void_p)]
     lib.wkf_tensor_clone.argtypes = [c_void_p, POINTER(c_void_p)]
@@ -475,6 +476,12 @@ class Tensor:
         h = c_void_p()
         _check(self._lib.wkf_tensor_reduce(self._h, REDUCE_OPS[name], int(dim), byref(h)))
         return self._new(h)
+
+    def reduce_into(self, name, dim, out):
+        """`self.<name>(dim)` written into `out` (a dense tensor that holds data) without any device allocation:
+        wkf_tensor_reduce_into.  Both tensors must be leaves; the kernels must have run once before."""
+        _check(self._lib.wkf_tensor_reduce_into(self._h, REDUCE_OPS[name], int(dim), out._h))
+        return out
 
     def sum(self, dim):
         return self._reduce("sum", dim)

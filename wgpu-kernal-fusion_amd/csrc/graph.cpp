@@ -219,6 +219,11 @@ NodeP Resolver::slice_through(const NodeP& n, size_t axis, size_t start, size_t 
   return result;
 }
 
+}  // namespace wkf
+// hip_ffi.cpp: the device's static scratch array as a buffer handle (a new reference) and its size
+wkf_buffer* wkf_scratch_(wkf_device* dev, size_t* bytes);
+namespace wkf {
+
 TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero) {
   TensorData td;
   td.device = dev_;
@@ -227,6 +232,24 @@ TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero
   wkf_buffer* b = nullptr;
   // padded_tensor_size, src/tensor.rs:775-783: a multiple of 4 bytes, at least 4.
   size_t bytes = std::max<size_t>(4, (td.layout.numel() * dtype_size(dt) + 3) & ~size_t(3));
+  if (noalloc_) {
+    // nothing is allocated: the result is the caller's tensor, a temporary is the device's static scratch array
+    if (zero) throw Error(WKF_ERR_UNSUPPORTED, "allocation-free call: the graph needs a zero-filled buffer");
+    if (!noalloc_->out_taken && shape == noalloc_->out.layout.shape && dt == noalloc_->out.dtype) {
+      noalloc_->out_taken = true;
+      return noalloc_->out;
+    }
+    size_t cap = 0;
+    wkf_buffer* sb = wkf_scratch_(dev_, &cap);
+    if (!sb) throw Error(WKF_ERR_HIP, "allocation-free call: the device has no scratch array");
+    td.buffer = BufRef(sb);
+    if (noalloc_->scratch_taken) throw Error(WKF_ERR_UNSUPPORTED, "allocation-free call: the graph needs more than one temporary");
+    if (bytes > cap)
+      throw Error(WKF_ERR_INVALID_ARG, "allocation-free call: the reduction needs " + std::to_string(bytes) +
+                                           " bytes of partial results, the static scratch array holds " + std::to_string(cap));
+    noalloc_->scratch_taken = true;
+    return td;
+  }
   check(wkf_buffer_alloc(dev_, bytes, zero ? 1 : 0, &b));
   td.buffer = BufRef(b);
   return td;
@@ -253,6 +276,9 @@ wkf_kernel* Resolver::kernel(const std::string& sig, const std::function<std::st
   wkf_kernel* cached = nullptr;
   check(wkf_module_find(dev_, sig.c_str(), &cached));
   if (cached) return cached;  // the hot path: no source text is built
+  if (noalloc_)
+    throw Error(WKF_ERR_INVALID_ARG, "allocation-free call: kernel '" + sig + "' is not loaded on this device (loading a code object "
+                "allocates); run wkf_tensor_reduce + wkf_tensor_materialize once on a tensor of this shape and dtype first");
   const std::string entry = entry_name(sig);
   const std::string src = "#define WKF_ENTRY " + entry + "\n" + make_body();
   {
@@ -272,7 +298,7 @@ wkf_kernel* Resolver::kernel(const std::string& sig, const std::function<std::st
 }
 
 void Resolver::record(LaunchRecord&& r, wkf_kernel* k, const std::vector<unsigned char>& args) {
-  if (st_.timing) check(wkf_timer_create(dev_, &r.timer));
+  if (st_.timing && !noalloc_) check(wkf_timer_create(dev_, &r.timer));
   int rc = wkf_launch(dev_, k, r.grid, r.block, 0, args.data(), args.size(), r.timer);
   if (rc != WKF_OK) {
     if (r.timer) wkf_timer_destroy(r.timer);

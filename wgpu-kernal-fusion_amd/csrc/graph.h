@@ -57,6 +57,14 @@ class Resolver {
   TensorData resolve_root(const NodeP& root);
   // Several tensors in one pass (shared sub-graphs once, sibling row reductions in one kernel).
   std::vector<TensorData> resolve_roots(const std::vector<NodeP>& roots);
+  // Allocation-free mode (wkf_tensor_reduce_into): the result goes into `out`, a temporary comes from the
+  // device's static scratch array (at most one, at most its size), and a kernel that this device has not loaded
+  // yet is an error instead of a compilation; no launch is timed.  Anything else the graph would allocate fails.
+  struct NoAlloc {
+    TensorData out;
+    bool out_taken = false, scratch_taken = false;
+  };
+  void set_noalloc(NoAlloc* na) { noalloc_ = na; }
 
  private:
   TensorData resolve(const NodeP& n);
@@ -128,6 +136,7 @@ class Resolver {
   wkf_kernel* kernel(const std::string& sig, const std::function<std::string()>& make_body);
 
   wkf_device* dev_;
+  NoAlloc* noalloc_ = nullptr;
   Settings st_;
   std::vector<LaunchRecord>* log_;
   std::set<const Node*> shared_;

@@ -78,6 +78,14 @@ std::string cache_dir() {
   return d;
 }
 
+// Scratch memory of the allocation-free entry point (wkf_tensor_reduce_into): the f32 partial sums of a reduction
+// that is folded in two launches.  A file-scope device array, so that nothing is allocated when the entry point
+// runs; every GPU this library is loaded on holds its own copy until the process ends.  Host code never passes the
+// array's name to a kernel: it is a host-side stand-in.  wkf_device_create asks the runtime for the device address
+// once per device (hipGetSymbolAddress) and keeps it.
+constexpr size_t kScratchBytes = size_t(1) << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
 size_t pool_bucket(size_t bytes) {
   if (bytes < 256) bytes = 256;
   if (bytes <= (1u << 20)) {
@@ -116,6 +124,9 @@ struct wkf_device {
   // events of destroyed timers, handed out again by wkf_timer_create: a timed launch costs two event
   // records, not two event creations and destructions
   std::vector<hipEvent_t> free_events;
+  // this device's copy of the file-scope scratch array (its address here, from hipGetSymbolAddress) behind a
+  // buffer handle that is never pooled or freed; on a plan-only device a host block of the same size
+  wkf_buffer* scratch_buf = nullptr;
 };
 
 struct wkf_buffer {
@@ -125,6 +136,7 @@ struct wkf_buffer {
   size_t capacity;
   std::atomic<int> refs;
   bool host_valid;  // plan-only devices: true once the host has uploaded contents
+  bool fixed = false;  // memory the buffer does not own (the static scratch array): never pooled, freed or counted
 };
 
 struct wkf_timer {
@@ -145,6 +157,15 @@ std::vector<void (*)(wkf_device*)> g_destroy_hooks;
 void wkf_add_destroy_hook_(void (*fn)(wkf_device*)) {
   std::lock_guard<std::mutex> lock(g_hooks_mu);
   g_destroy_hooks.push_back(fn);
+}
+
+// The per-device scratch array of the allocation-free entry point as a buffer handle (a new reference: release it
+// like any other), and its size.  The layers above use it in place of an allocated temporary.
+wkf_buffer* wkf_scratch_(wkf_device* dev, size_t* bytes) {
+  if (!dev || !dev->scratch_buf) return nullptr;
+  if (bytes) *bytes = kScratchBytes;
+  dev->scratch_buf->refs.fetch_add(1, std::memory_order_relaxed);
+  return dev->scratch_buf;
 }
 
 extern "C" {
@@ -185,6 +206,17 @@ int wkf_device_create(int ordinal, wkf_device** out) {
     return fail(WKF_ERR_UNSUPPORTED, "wkf_device_create: kernels are written for gfx950, device is " + arch);
   }
   d->cache_path = cache_dir();
+  {
+    // the device address of THIS device's copy of the scratch array (the device is current: hipSetDevice above)
+    void* sp = nullptr;
+    hipError_t ge = hipGetSymbolAddress(&sp, HIP_SYMBOL(scratch));
+    if (ge != hipSuccess || !sp) {
+      hipStreamDestroy(d->stream);
+      delete d;
+      return fail(WKF_ERR_HIP, std::string("hipGetSymbolAddress(scratch): ") + hipGetErrorString(ge));
+    }
+    d->scratch_buf = new wkf_buffer{d, sp, kScratchBytes, kScratchBytes, {1}, false, true};
+  }
   *out = d;
   return WKF_OK;
 }
@@ -202,6 +234,12 @@ int wkf_device_create_planner(wkf_device** out) {
   d->props.total_mem_bytes = size_t(288) << 30;
   snprintf(d->props.arch, sizeof(d->props.arch), "gfx950");
   d->cache_path = cache_dir();
+  void* sp = malloc(kScratchBytes);
+  if (!sp) {
+    delete d;
+    return fail(WKF_ERR_OOM, "wkf_device_create_planner: host allocation failed");
+  }
+  d->scratch_buf = new wkf_buffer{d, sp, kScratchBytes, kScratchBytes, {1}, false, true};
   *out = d;
   return WKF_OK;
 }
@@ -255,6 +293,10 @@ static void destroy_now(wkf_device* dev) {
   for (auto& kv : dev->kernels) {
     if (kv.second->module) hipModuleUnload(kv.second->module);
     delete kv.second;
+  }
+  if (dev->scratch_buf) {
+    if (dev->planner) free(dev->scratch_buf->ptr);
+    delete dev->scratch_buf;
   }
   for (hipEvent_t e : dev->free_events) hipEventDestroy(e);
   if (dev->stream) hipStreamDestroy(dev->stream);
@@ -324,6 +366,7 @@ void wkf_buffer_retain(wkf_buffer* buf) {
 void wkf_buffer_release(wkf_buffer* buf) {
   if (!buf) return;
   if (buf->refs.fetch_sub(1, std::memory_order_acq_rel) != 1) return;
+  if (buf->fixed) return;  // the device keeps its own reference until it is destroyed; nothing to pool or free
   wkf_device* dev = buf->dev;
   bool last = false;
   {

@@ -6,6 +6,7 @@
 #include <cmath>
 #include <cstring>
 #include <mutex>
+#include <sstream>
 #include <unordered_map>
 
 #include "graph.h"
@@ -554,6 +555,32 @@ int wkf_tensor_reduce(const wkf_tensor* t, int reduce_op, size_t axis, wkf_tenso
     need(out, "wkf_tensor_reduce");
     if (reduce_op < 0 || reduce_op > 3) invalid("wkf_tensor_reduce: unknown reduction");
     *out = wrap(t->dev, n_reduce(t->node, ReduceOp(reduce_op), axis));
+  });
+}
+
+int wkf_tensor_reduce_into(const wkf_tensor* t, int reduce_op, size_t axis, wkf_tensor* out) {
+  return guarded([&] {
+    need(t, "wkf_tensor_reduce_into");
+    need(out, "wkf_tensor_reduce_into");
+    if (reduce_op < 0 || reduce_op > 3) invalid("wkf_tensor_reduce_into: unknown reduction");
+    if (t->dev != out->dev) invalid("wkf_tensor_reduce_into: tensors live on different devices");
+    // both tensors hold data already (leaves): nothing below them needs a kernel or a buffer
+    if (t->node->kind != NodeKind::Tensor || out->node->kind != NodeKind::Tensor)
+      invalid("wkf_tensor_reduce_into: the input and the output must be tensors that hold data (wkf_tensor_new), not lazy expressions");
+    if (!t->node->data.layout.is_contiguous() || !out->node->data.layout.is_contiguous())
+      invalid("wkf_tensor_reduce_into: the input and the output must be dense");
+    NodeP rn = n_reduce(t->node, ReduceOp(reduce_op), axis);  // checks the axis; shape and dtype of the result
+    if (out->node->shape != rn->shape || out->node->dtype != rn->dtype)
+      invalid("wkf_tensor_reduce_into: the output must have the input's shape without the reduced axis, and its dtype");
+    if (wkf_buffer_ptr(out->node->data.buffer.get()) == wkf_buffer_ptr(t->node->data.buffer.get()))
+      invalid("wkf_tensor_reduce_into: the output shares the input's buffer");
+    Resolver::NoAlloc na;
+    na.out = out->node->data;
+    Resolver res(t->dev, settings_for(t->dev), nullptr);
+    res.set_noalloc(&na);
+    TensorData got = res.resolve_root(rn);
+    if (got.buffer.get() != na.out.buffer.get())
+      throw Error(WKF_ERR_UNSUPPORTED, "wkf_tensor_reduce_into: the result was not written to the output tensor");
   });
 }
 
