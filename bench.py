@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Benchmark of the fused hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-detail] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-detail] [--no-cpu] [--only c1,c5,f16]
+    python bench.py --profile c5_f16 [--launches N]     (one workload only, for rocprofv3)
 
 Prints ONE JSON line.  The headline (`value`) is BASELINE.json's metric on its
 configuration 2: one step = the two fused row-reduce kernels of a softmax,
@@ -11,7 +12,9 @@ over several input tensors so that the 256 MB Infinity Cache cannot serve them.
 `roofline` is the dominant kernel (the exp-sum reduce) timed with hipEvent pairs
 on the stream it runs on; `cpu_baseline` is the CPU port of the reference's
 decomposition (oracle/port.c) on this box's host cores; `all_configs` carries
-every BASELINE configuration (GB/s or TFLOP/s and the fraction of the roofline).
+every BASELINE configuration (GB/s or TFLOP/s, the fraction of its roofline, the median and the minimum of the
+per-launch times after at least 100 warm launches, and the CPU port timed on a bounded sample of the same
+configuration), plus f16 rows of the memory-bound kernels.
 
 Everything runs on one GPU: `--gpus N` with N > 1 is refused.
 """
@@ -56,11 +59,14 @@ def rope_tables(seq, dim, theta=10000.0):
 
 
 class Workload:
-    """`variants`: the same expression over different input tensors (rotated step by step)."""
+    """`variants`: the same expression over different input tensors (rotated step by step).
+    `cpu`: (callable, work, text) -- the CPU port of the same computation on a bounded sample of it: calling the
+    callable runs the sample once, `work` is the sample's algorithmic bytes or flops, `text` says what it was."""
 
-    def __init__(self, name, variants, work, unit, peak, dtype="f32", joint=None):
+    def __init__(self, name, variants, work, unit, peak, dtype="f32", joint=None, cpu=None):
         self.name, self.variants, self.work, self.unit, self.peak, self.dtype = name, variants, work, unit, peak, dtype
         self.joint = joint  # the package's materialize_many: the tensors of a step are materialised in ONE pass
+        self.cpu = cpu
 
     def step(self, i):
         """Launches step i; returns the tensors whose kernel records describe it."""
@@ -74,23 +80,26 @@ class Workload:
 
 
 def measure_kernels(dev, wl, steps, warmup):
-    """Per-kernel GPU time (hipEvent pair around each launch), averaged over `steps` steps."""
+    """Per-kernel GPU time (hipEvent pair around each launch) over `steps` steps after `warmup` untimed ones:
+    the median and the minimum per kernel, and of the step's total."""
     dev.set_timing(True)
     for i in range(warmup):
         wl.step(i)
     dev.sync()
-    sums, kinds, details = None, None, None
+    samples, kinds, details = [], None, None
     for i in range(steps):
-        ns = []
         ks = []
         for t in wl.step(i):
             ks += t.kernels()
-        ns = np.array([k.elapsed_ns for k in ks], dtype=np.float64)
-        sums = ns if sums is None else sums + ns
+        samples.append([k.elapsed_ns for k in ks])
         kinds = [k.kind for k in ks]
         details = [k.detail for k in ks]
-    avg = sums / steps
-    return [{"kind": k, "detail": d, "us": round(float(a) / 1e3, 2)} for k, d, a in zip(kinds, details, avg)]
+    arr = np.array(samples, dtype=np.float64) / 1e3  # [step][kernel] in us
+    med, mn = np.median(arr, axis=0), arr.min(axis=0)
+    total = arr.sum(axis=1)
+    kernels = [{"kind": k, "detail": d, "us": round(float(a), 2), "min_us": round(float(b), 2)}
+               for k, d, a, b in zip(kinds, details, med, mn)]
+    return kernels, round(float(np.median(total)), 2), round(float(total.min()), 2)
 
 
 def measure_batch(w, dev, wl, steps, warmup):
@@ -133,69 +142,197 @@ def measure_wall(dev, wl, steps, warmup):
         dev.set_timing(True)
 
 
-def summarise(wl, kernels, wall_s, steps, batch_us):
-    gpu_us = sum(k["us"] for k in kernels)
+def summarise(wl, measured, wall_s, steps, batch_us):
+    kernels, med_us, min_us = measured
     scale = 1e-3 if wl.unit == "GB/s" else 1e-6  # bytes/us -> GB/s ; flop/us -> TFLOP/s
+    rate = lambda us: round(wl.work / us * scale, 1) if us else None
+    frac = lambda us: round(wl.work / us * scale / wl.peak, 4) if us else None
+    dom = max(kernels, key=lambda k: k["us"])
+    # the roofline of this configuration: its dominant kernel, timed without per-launch events when a batch figure
+    # exists (one hipEvent pair around `steps` back-to-back steps on the library's stream)
+    step_us = batch_us if batch_us else med_us
     return {"name": wl.name, "dtype": wl.dtype, "unit": wl.unit, "work_per_step": wl.work,
-            "kernels": kernels, "gpu_us_per_step": round(gpu_us, 2),
-            "achieved": round(wl.work / gpu_us * scale, 1), "peak": wl.peak,
-            "frac": round(wl.work / gpu_us * scale / wl.peak, 4), "batch_us_per_step": batch_us,
-            "batch_achieved": round(wl.work / batch_us * scale, 1) if batch_us else None,
-            "batch_frac": round(wl.work / batch_us * scale / wl.peak, 4) if batch_us else None,
+            "kernels": kernels, "median_us_per_step": med_us, "min_us_per_step": min_us,
+            "achieved": rate(med_us), "peak": wl.peak, "frac": frac(med_us), "min_frac": frac(min_us),
+            "batch_us_per_step": batch_us, "batch_achieved": rate(batch_us), "batch_frac": frac(batch_us),
+            "roofline": {"bound": "hbm" if wl.unit == "GB/s" else "mfma", "kernel": dom["kind"] + " " + dom["detail"],
+                         "kernels_per_step": len(kernels), "avg_us": step_us, "achieved": rate(step_us), "peak": wl.peak,
+                         "unit": wl.unit, "frac": frac(step_us)},
             "wall_ms_per_step": round(wall_s / steps * 1e3, 4),
             "wall_rate": round(wl.work * steps / wall_s * (1e-9 if wl.unit == "GB/s" else 1e-12), 1)}
 
 
-def build_workloads(w, dev, seeded, which):
+def build_workloads(w, dev, seeded, which, with_cpu=False):
+    """The BASELINE configurations (c1..c5) and the f16 rows of the memory-bound kernels (f16) as workloads.
+    with_cpu: also prepare the CPU port of each configuration (oracle/port.c) on a bounded sample of its inputs."""
     T = w.Tensor
     out = {}
+    port = None
+    if with_cpu:
+        from oracle import port as port_mod
+        port_mod.load()
+        port = port_mod
+
+    def cpu_of(fn, work, text):
+        return (fn, work, text) if port is not None else None
+
     if "c2" in which:
-        xs = [T.new(dev, seeded(2, r, (8192, 8192), "normal")) for r in range(4)]
+        hosts = [seeded(2, r, (8192, 8192), "normal") for r in range(4)]
+        xs = [T.new(dev, h) for h in hosts]
+        h0 = hosts[0]
+        del hosts
+        o = np.empty(8192, dtype=np.float32)
+        both = cpu_of(lambda: (port.row_max(h0, o), port.row_sum_exp_sub(h0, 1.0, o)), 2 * 268468224, "the full step")
         out["c2"] = Workload("config2: row max(x) + row sum(exp(x-1)), f32 [8192,8192]",
-                             [[x.max(1), (x.clone() - 1.0).exp().sum(1)] for x in xs], 2 * 268468224, "GB/s", HBM_PEAK_GBS)
+                             [[x.max(1), (x.clone() - 1.0).exp().sum(1)] for x in xs], 2 * 268468224, "GB/s", HBM_PEAK_GBS, cpu=both)
         # the same two results from ONE pass over the matrix (the reference lists this fusion as to-do, README.md:20):
         # algorithmic bytes = the matrix once + both result vectors
         out["c2_one_pass"] = Workload("config2 in one pass: row max(x) and row sum(exp(x-1)) together, f32 [8192,8192]",
                                       [[x.max(1), (x.clone() - 1.0).exp().sum(1)] for x in xs], 8192 * 8192 * 4 + 2 * 8192 * 4,
                                       "GB/s", HBM_PEAK_GBS, joint=w.materialize_many)
-        out["c2a"] = Workload("config2a: row max(x), f32 [8192,8192]", [[x.max(1)] for x in xs], 268468224, "GB/s", HBM_PEAK_GBS)
+        out["c2a"] = Workload("config2a: row max(x), f32 [8192,8192]", [[x.max(1)] for x in xs], 268468224, "GB/s", HBM_PEAK_GBS,
+                              cpu=cpu_of(lambda: port.row_max(h0, o), 268468224, "the full kernel"))
         out["c2b"] = Workload("config2b: row sum(exp(x-1)), f32 [8192,8192]", [[(x.clone() - 1.0).exp().sum(1)] for x in xs],
-                              268468224, "GB/s", HBM_PEAK_GBS)
+                              268468224, "GB/s", HBM_PEAK_GBS,
+                              cpu=cpu_of(lambda: port.row_sum_exp_sub(h0, 1.0, o), 268468224, "the full kernel"))
     if "c1" in which:
-        xs = [T.new(dev, seeded(1, r, (4096, 4096), "uniform")) for r in range(8)]
+        hosts = [seeded(1, r, (4096, 4096), "uniform") for r in range(8)]
+        xs = [T.new(dev, h) for h in hosts]
+        h1 = hosts[0]
+        del hosts
+        y1 = np.empty_like(h1)
         out["c1"] = Workload("config1: exp(sin(x*2+1)), f32 [4096,4096]", [[((x * 2.0) + 1.0).sin().exp()] for x in xs],
-                             134217728, "GB/s", HBM_PEAK_GBS)
+                             134217728, "GB/s", HBM_PEAK_GBS, cpu=cpu_of(lambda: port.c1(h1, y1), 134217728, "the full tensor"))
     if "c3" in which:
         variants = []
-        bias = T.new(dev, seeded(3, 2, (4096,), "normal", std=0.02))
+        hb = seeded(3, 2, (4096,), "normal", std=0.02)
+        bias = T.new(dev, hb)
         bias3 = bias.broadcast([1024, 4096]).broadcast([32, 1024, 4096])
+        keep = None
         for r in range(2):
-            a = T.new(dev, seeded(3, 4 * r, (32, 1024, 4096), "uniform"))
-            b = T.new(dev, seeded(3, 4 * r + 1, (32, 1024, 4096), "uniform"))
+            ha = seeded(3, 4 * r, (32, 1024, 4096), "uniform")
+            hbb = seeded(3, 4 * r + 1, (32, 1024, 4096), "uniform")
+            a, b = T.new(dev, ha), T.new(dev, hbb)
+            if r == 0 and port is not None:
+                keep = (np.ascontiguousarray(ha[:8]), np.ascontiguousarray(hbb[:8]))  # 8 of the 32 slabs
             variants.append([a.silu() * (b + bias3)])
-        out["c3"] = Workload("config3: silu(a)*(b+bias), f32 [32,1024,4096]", variants, 1610629120, "GB/s", HBM_PEAK_GBS)
+        cpu3 = None
+        if keep is not None:
+            t1, t2 = np.empty_like(keep[0]), np.empty_like(keep[0])
+            cpu3 = cpu_of(lambda: port.c3(keep[0], keep[1], hb, t1, t2), 1610629120 // 4,
+                          "8 of the 32 [1024,4096] slabs, the reference's three passes (silu, add, mul)")
+        out["c3"] = Workload("config3: silu(a)*(b+bias), f32 [32,1024,4096]", variants, 1610629120, "GB/s", HBM_PEAK_GBS, cpu=cpu3)
     if "c4" in which:
-        w4 = T.new(dev, seeded(4, 1, (4096,), "normal", mean=1.0, std=0.02))
-        xs = [T.new(dev, seeded(4, 8 + r, (2048, 4096), "normal")) for r in range(8)]
-        out["c4_rmsnorm"] = Workload("config4: RMSNorm f32 [2048,4096]", [[x.layer_norm(w4, 1e-5)] for x in xs], 67125248, "GB/s", HBM_PEAK_GBS)
+        hw = seeded(4, 1, (4096,), "normal", mean=1.0, std=0.02)
+        w4 = T.new(dev, hw)
+        hosts = [seeded(4, 8 + r, (2048, 4096), "normal") for r in range(8)]
+        xs = [T.new(dev, h) for h in hosts]
+        hx = hosts[0]
+        del hosts
+        out["c4_rmsnorm"] = Workload("config4: RMSNorm f32 [2048,4096]", [[x.layer_norm(w4, 1e-5)] for x in xs], 67125248, "GB/s",
+                                     HBM_PEAK_GBS, cpu=cpu_of(lambda: port.rmsnorm(hx, hw, 1e-5), 67125248, "the full tensor"))
         cos, sin = rope_tables(2048, 128)
         tc, ts = T.new(dev, cos), T.new(dev, sin)
-        qs = [T.new(dev, seeded(4, 16 + r, (32, 2048, 128), "normal")) for r in range(8)]
-        out["c4_rope"] = Workload("config4: RoPE f32 [32,2048,128]", [[q.rope(tc, ts)] for q in qs], 69206016, "GB/s", HBM_PEAK_GBS)
-        ss = [T.new(dev, seeded(4, 24 + r, (32, 2048, 2048), "normal")) for r in range(2)]
-        out["c4_softmax"] = Workload("config4: softmax f32 [32,2048,2048]", [[s.softmax_last_dim()] for s in ss], 1073741824, "GB/s", HBM_PEAK_GBS)
+        hosts = [seeded(4, 16 + r, (32, 2048, 128), "normal") for r in range(8)]
+        qs = [T.new(dev, h) for h in hosts]
+        hq = hosts[0]
+        del hosts
+        cf, sf = np.ascontiguousarray(np.concatenate([cos, cos], 1)), np.ascontiguousarray(np.concatenate([sin, sin], 1))
+        out["c4_rope"] = Workload("config4: RoPE f32 [32,2048,128]", [[q.rope(tc, ts)] for q in qs], 69206016, "GB/s", HBM_PEAK_GBS,
+                                  cpu=cpu_of(lambda: port.rope(hq, cf, sf), 69206016, "the full tensor"))
+        hosts = [seeded(4, 24 + r, (32, 2048, 2048), "normal") for r in range(2)]
+        ss = [T.new(dev, h) for h in hosts]
+        hs = np.ascontiguousarray(hosts[0][:8])
+        del hosts
+        out["c4_softmax"] = Workload("config4: softmax f32 [32,2048,2048]", [[s.softmax_last_dim()] for s in ss], 1073741824, "GB/s",
+                                     HBM_PEAK_GBS, cpu=cpu_of(lambda: port.softmax_rows(hs), 1073741824 // 4,
+                                                              "8 of the 32 heads, the reference's passes (max, exp-sum, divide)"))
     if "c5" in which:
-        a32 = T.new(dev, seeded(5, 0, (4096, 4096), "normal", std=0.02))
-        b32 = T.new(dev, seeded(5, 1, (4096, 4096), "normal", std=0.02))
-        out["c5_f32"] = Workload("config5a: GEMM f32 4096^3", [[a32.mat_mul(b32)]], 137438953472, "TFLOP/s", F32_MFMA_PEAK_TFLOPS)
+        ha = seeded(5, 0, (4096, 4096), "normal", std=0.02)
+        hb5 = seeded(5, 1, (4096, 4096), "normal", std=0.02)
+        a32, b32 = T.new(dev, ha), T.new(dev, hb5)
+        rows = np.ascontiguousarray(ha[:256])
+        gemm_cpu = cpu_of(lambda: port.gemm_f32(rows, hb5), 2 * 256 * 4096 * 4096, "256 of the 4096 rows of A against all of B, f32")
+        out["c5_f32"] = Workload("config5a: GEMM f32 4096^3", [[a32.mat_mul(b32)]], 137438953472, "TFLOP/s", F32_MFMA_PEAK_TFLOPS,
+                                 cpu=gemm_cpu)
         a16 = T.new(dev, seeded(5, 0, (4096, 4096), "normal", dtype=np.float16, std=0.02))
         b16 = T.new(dev, seeded(5, 1, (4096, 4096), "normal", dtype=np.float16, std=0.02))
-        out["c5_f16"] = Workload("config5b: GEMM f16 4096^3", [[a16.mat_mul(b16)]], 137438953472, "TFLOP/s", F16_MFMA_PEAK_TFLOPS, "f16")
+        gemm_cpu16 = cpu_of(lambda: port.gemm_f32(rows, hb5), 2 * 256 * 4096 * 4096,
+                            "256 of the 4096 rows of A against all of B, in f32 arithmetic (the port has no f16 path)")
+        out["c5_f16"] = Workload("config5b: GEMM f16 4096^3", [[a16.mat_mul(b16)]], 137438953472, "TFLOP/s", F16_MFMA_PEAK_TFLOPS, "f16",
+                                 cpu=gemm_cpu16)
         am = T.new(dev, seeded(5, 2, (2048, 4096), "normal", dtype=np.float16, std=0.02))
-        bm = T.new(dev, seeded(5, 3, (4096, 11008), "normal", dtype=np.float16, std=0.02))
+        hbm = seeded(5, 3, (4096, 11008), "normal", dtype=np.float16, std=0.02)
+        bm = T.new(dev, hbm)
+        mlp_cpu = None
+        if port is not None:
+            hbm32 = hbm.astype(np.float32)
+            mlp_cpu = cpu_of(lambda: port.gemm_f32(rows, hbm32), 2 * 256 * 4096 * 11008,
+                             "256 rows against all of the [4096,11008] weight, in f32 arithmetic (the port has no f16 path)")
+        del hbm
         out["c5_mlp"] = Workload("config5c: GEMM f16 [2048x4096]x[4096x11008]", [[am.mat_mul(bm)]], 184683593728, "TFLOP/s",
-                                 F16_MFMA_PEAK_TFLOPS, "f16")
+                                 F16_MFMA_PEAK_TFLOPS, "f16", cpu=mlp_cpu)
+    if "f16" in which:
+        # the f16 forms of the memory-bound kernels (no BASELINE configuration names them; no CPU figure)
+        F16 = np.float16
+        xs = [T.new(dev, seeded(2, r, (8192, 8192), "normal", dtype=F16)) for r in range(4)]
+        out["f16_c2"] = Workload("f16: row max(x) + row sum(exp(x-1)), f16 [8192,8192]",
+                                 [[x.max(1), (x.clone() - 1.0).exp().sum(1)] for x in xs], 2 * (8192 * 8192 * 2 + 8192 * 2), "GB/s",
+                                 HBM_PEAK_GBS, "f16")
+        out["f16_sum"] = Workload("f16: row sum(x), f16 [8192,8192]", [[x.sum(1)] for x in xs], 8192 * 8192 * 2 + 8192 * 2, "GB/s",
+                                  HBM_PEAK_GBS, "f16")
+        out["f16_map"] = Workload("f16: exp(sin(x*2+1)), f16 [8192,8192]", [[((x * 2.0) + 1.0).sin().exp()] for x in xs],
+                                  2 * 8192 * 8192 * 2, "GB/s", HBM_PEAK_GBS, "f16")
+        x32 = [T.new(dev, seeded(2, r, (8192, 8192), "normal")) for r in range(2)]
+        out["f16_cast"] = Workload("cast f32 -> f16, [8192,8192]", [[x.cast(w.F16)] for x in x32], 8192 * 8192 * 6, "GB/s",
+                                   HBM_PEAK_GBS, "f32->f16")
+        ss = [T.new(dev, seeded(4, 24 + r, (32, 2048, 2048), "normal", dtype=F16)) for r in range(2)]
+        out["f16_softmax"] = Workload("f16: softmax f16 [32,2048,2048]", [[s_.softmax_last_dim()] for s_ in ss], 2 * 32 * 2048 * 2048 * 2,
+                                      "GB/s", HBM_PEAK_GBS, "f16")
+        w16 = T.new(dev, seeded(4, 1, (4096,), "normal", dtype=F16, mean=1.0, std=0.02))
+        x16 = [T.new(dev, seeded(4, 8 + r, (2048, 4096), "normal", dtype=F16)) for r in range(8)]
+        out["f16_rmsnorm"] = Workload("f16: RMSNorm f16 [2048,4096]", [[x.layer_norm(w16, 1e-5)] for x in x16],
+                                      2 * 2048 * 4096 * 2 + 4096 * 2, "GB/s", HBM_PEAK_GBS, "f16")
     return out
+
+
+def time_cpu(cpu, budget_s=3.0):
+    """Median seconds of the CPU port's sample over at least 2 runs (one untimed first), within about `budget_s`."""
+    fn, work, text = cpu
+    fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 2 or (time.perf_counter() < t_end and len(times) < 20):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return float(np.median(times)), len(times)
+
+
+def cpu_row(wl):
+    """The `cpu_baseline` object of one configuration: oracle/port.c on the host cores, on a bounded sample."""
+    from oracle import port
+    med, n = time_cpu(wl.cpu)
+    scale = 1e-9 if wl.unit == "GB/s" else 1e-12
+    return {"value": round(wl.cpu[1] / med * scale, 3), "unit": wl.unit, "cores": port.threads(), "kind": "port",
+            "sample": f"{wl.cpu[2]}; median of {n} runs of oracle/port.c (OpenMP)"}
+
+
+def reference_cpu_path():
+    """Run-time probe for what the reference's own CPU path needs (cargo / rustc and a Vulkan CPU adapter such as
+    lavapipe): reported next to the CPU port's figures."""
+    import glob
+    import shutil
+    icds = []
+    for d in ("/usr/share/vulkan/icd.d", "/etc/vulkan/icd.d", "/usr/local/share/vulkan/icd.d"):
+        icds += glob.glob(os.path.join(d, "*.json"))
+    lvp = [p for p in icds if "lvp" in os.path.basename(p) or "lavapipe" in os.path.basename(p)]
+    probe = {"cargo": shutil.which("cargo"), "rustc": shutil.which("rustc"), "vulkan_icds": icds, "lavapipe_icd": lvp[:1] or None,
+             "reference_checkout": os.path.isdir("/root/reference")}
+    ok = bool(probe["cargo"] and probe["rustc"] and lvp and probe["reference_checkout"])
+    return {"available": ok, "probe": probe,
+            "note": "the reference's wgpu path on a CPU adapter needs cargo + rustc + a Vulkan CPU ICD + its checkout; "
+                    + ("all present, but this benchmark does not drive it" if ok else "unavailable on this machine, so the CPU figures are oracle/port.c")}
 
 
 def copy_ceiling(w, dev):
@@ -203,29 +340,28 @@ def copy_ceiling(w, dev):
     x = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32))
     t = x.resize([1 << 28])  # resize to the same shape = one dense copy kernel
     wl = Workload("copy", [[t]], 2 * (1 << 30), "GB/s", HBM_PEAK_GBS)
-    k = measure_kernels(dev, wl, 10, 3)
-    return round(wl.work / k[0]["us"] * 1e-3, 1)
+    k, med, _ = measure_kernels(dev, wl, 10, 3)
+    return round(wl.work / med * 1e-3, 1)
 
 
-def cpu_baseline(seeded):
-    """The CPU port (oracle/port.c), timed on this box's host cores: config 2, full size."""
+def cpu_baseline(wl):
+    """The CPU port (oracle/port.c) of the headline configuration, timed on this box's host cores at full size."""
     from oracle import port
-    port.load()
-    x = seeded(2, 0, (8192, 8192), "normal")
-    out = np.empty(8192, dtype=np.float32)
-    port.row_max(x, out)
-    port.row_sum_exp_sub(x, 1.0, out)
+    fn = wl.cpu[0]
+    fn()
     times = []
-    t_end = time.perf_counter() + 15.0
+    t_end = time.perf_counter() + 12.0
     while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 40):
         t0 = time.perf_counter()
-        port.row_max(x, out)
-        port.row_sum_exp_sub(x, 1.0, out)
+        fn()
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
-    return {"value": round(2 * 268468224 / med * 1e-9, 2), "unit": "GB/s", "cores": port.threads(), "kind": "port",
+    return {"value": round(wl.cpu[1] / med * 1e-9, 2), "unit": "GB/s", "cores": port.threads(), "kind": "port",
             "sample": f"the full config-2 step (row max + row sum(exp(x-1)) on f32 [8192,8192]), median of {len(times)} runs, "
-                      "oracle/port.c with OpenMP (the reference's wgpu path cannot run: no Rust toolchain, no Vulkan ICD)"}
+                      "oracle/port.c with OpenMP"}
+
+
+GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16")
 
 
 def plan_only(w):
@@ -240,7 +376,7 @@ def plan_only(w):
     copy = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32)).resize([1 << 28])
     copy.materialize()
     del copy
-    for gname in ("c1", "c2", "c3", "c4", "c5"):
+    for gname in GROUPS:
         wls = build_workloads(w, dev, zeros, {gname})
         for one in wls.values():
             for mode in ((w.FUSION_TREE, w.FUSION_REFERENCE) if gname in ("c3", "c4") else (w.FUSION_TREE,)):
@@ -253,16 +389,39 @@ def plan_only(w):
                       "kernels_from_disk_cache": after["disk_hits"] - before["disk_hits"]}))
 
 
+def profile_one(w, dev, seeded, key, launches):
+    """`--profile KEY`: nothing but `launches` steps of one workload (after 10 untimed ones), for a profiler run
+    (rocprofv3 --kernel-trace --stats / --pmc ... -- python3 bench.py --profile KEY)."""
+    group = key.split("_")[0]
+    if key == "copy":
+        x = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32))
+        wl = Workload("copy 1 GiB -> 1 GiB", [[x.resize([1 << 28])]], 2 * (1 << 30), "GB/s", HBM_PEAK_GBS)
+    else:
+        wls = build_workloads(w, dev, seeded, {group})
+        if key not in wls:
+            sys.exit(f"bench.py --profile: unknown workload {key!r}; one of copy, " + ", ".join(
+                k for g in GROUPS for k in build_workloads(w, w.Device.planner(), lambda *a, **kw: np.zeros(a[2], dtype=kw.get("dtype", np.float32)), {g})))
+        wl = wls[key]
+    us = measure_batch(w, dev, wl, launches, 10)
+    scale = 1e-3 if wl.unit == "GB/s" else 1e-6
+    print(json.dumps({"profile": key, "name": wl.name, "launches": launches, "us_per_step": round(us, 2),
+                      "achieved": round(wl.work / us * scale, 1), "unit": wl.unit, "frac": round(wl.work / us * scale / wl.peak, 4),
+                      "work_per_step": wl.work}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="only the headline configuration")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5 for the detail table")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
+    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16 for the detail table")
     ap.add_argument("--plan-only", action="store_true",
                     help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
+    ap.add_argument("--profile", default="", help="run one workload only (copy, c1, c2a, c2b, c3, c4_rmsnorm, c4_rope, c4_softmax, "
+                                                  "c5_f32, c5_f16, c5_mlp, f16_*), for a profiler")
+    ap.add_argument("--launches", type=int, default=30, help="timed steps of --profile")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every kernel, no collectives); --gpus must be 1.")
@@ -277,14 +436,18 @@ def main():
         return
     dev = w.Device.new(0)
     props = dev.props()
+    if args.profile:
+        profile_one(w, dev, seeded, args.profile, args.launches)
+        return
     if args.only == "copy":
         # calibration run for the rocprofv3 counters: nothing but the 1 GiB -> 1 GiB copy kernel
         print(json.dumps({"copy_kernel_GBs": copy_ceiling(w, dev), "bytes_read": 1 << 30, "bytes_written": 1 << 30}))
         return
 
-    head = build_workloads(w, dev, seeded, {"c2"})
+    with_cpu = not args.no_cpu
+    head = build_workloads(w, dev, seeded, {"c2"}, with_cpu)
     wl = head["c2"]
-    kernels = measure_kernels(dev, wl, args.steps, args.warmup)
+    kernels, _, _ = measure_kernels(dev, wl, args.steps, args.warmup)
     wall = measure_wall(dev, wl, args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
     value = wl.work * args.steps / wall * 1e-9
@@ -304,50 +467,62 @@ def main():
         "config": {"workload": wl.name, "seed": "SplitMix64 0x5EED0020+r", "rotating_inputs": len(wl.variants),
                    "kernels_per_step": len(kernels), "algorithmic_bytes_per_step": wl.work,
                    "kernel_us": {"row_max": round(max_us, 2), "row_sum_exp": round(dom_us, 2),
-                                 "per_launch_event_pairs": [k["us"] for k in kernels]},
+                                 "per_launch_event_pairs_median": [k["us"] for k in kernels]},
                    "device": props.arch.decode(), "compute_units": props.compute_units, "clock_khz": props.clock_khz},
         "roofline": {"bound": "hbm", "achieved": round(268468224 / dominant["us"] * 1e-3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(268468224 / dominant["us"] * 1e-3 / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, calibrated "
+                                       "with the copy kernel, taken in a profiler run of its own; not measured by this run",
                      "kernel": dominant["kind"] + " " + dominant["detail"], "avg_us": dominant["us"],
                      "algorithmic_bytes_per_launch": 268468224},
         "value_frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
     }
+    result["cpu_baseline"] = cpu_baseline(wl) if with_cpu else None
+    result["reference_cpu_path"] = reference_cpu_path()
     del head, wl
     dev.trim()
-    if not args.no_cpu:
-        result["cpu_baseline"] = cpu_baseline(seeded)
-    else:
-        result["cpu_baseline"] = None
     if not args.no_detail:
         detail = []
         result["copy_kernel_GBs"] = copy_ceiling(w, dev)
         dev.trim()
-        groups = [g for g in ("c1", "c2", "c3", "c4", "c5") if not args.only or g in args.only.split(",")]
-        steps = max(10, min(args.steps, 50))
+        groups = [g for g in GROUPS if not args.only or g in args.only.split(",")]
+        steps = max(20, min(args.steps, 50))
+        warm = 100  # launches before anything is timed: the first launches after an idle GPU run slower (clock ramp)
         for gname in groups:
-            wls = build_workloads(w, dev, seeded, {gname})
+            wls = build_workloads(w, dev, seeded, {gname}, with_cpu)
             for key, one in wls.items():
                 if key == "c2":
                     continue
-                ks = measure_kernels(dev, one, steps, 5)
+                measured = measure_kernels(dev, one, steps, warm)
                 wall_s = measure_wall(dev, one, steps, 5)
                 batch_us = round(measure_batch(w, dev, one, steps, 5), 2)
-                detail.append(summarise(one, ks, wall_s, steps, batch_us))
+                row = summarise(one, measured, wall_s, steps, batch_us)
+                row["key"] = key
+                row["cpu_baseline"] = cpu_row(one) if (with_cpu and one.cpu) else None
+                detail.append(row)
                 if gname in ("c3", "c4"):
                     # the same graph under the reference's own fusion rules (its kernel decomposition):
                     # same algorithmic work, more passes over memory
                     dev.set_fusion(w.FUSION_REFERENCE)
                     try:
-                        ks = measure_kernels(dev, one, steps, 5)
+                        measured = measure_kernels(dev, one, steps, 20)
                         wall_s = measure_wall(dev, one, steps, 5)
-                        row = summarise(one, ks, wall_s, steps, None)
+                        row = summarise(one, measured, wall_s, steps, None)
+                        row["key"] = key + "_reference_rules"
                         row["name"] += " -- reference kernel decomposition"
+                        row["cpu_baseline"] = None
                         detail.append(row)
                     finally:
                         dev.set_fusion(w.FUSION_TREE)
             del wls
             dev.trim()
         result["all_configs"] = detail
+        # the configuration furthest below its roofline (BASELINE configurations only, as this library fuses them)
+        own = [r for r in detail if r["key"][0] == "c" and not r["key"].endswith("_reference_rules") and r["key"] != "c2_one_pass"]
+        if own:
+            worst = min(own, key=lambda r: r["roofline"]["frac"])
+            result["worst_config"] = {"name": worst["name"], "frac": worst["roofline"]["frac"], "achieved": worst["roofline"]["achieved"],
+                                      "unit": worst["unit"]}
     print(json.dumps(result))
 
 
