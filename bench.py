@@ -399,14 +399,168 @@ def profile_one(w, dev, seeded, key, launches):
     else:
         wls = build_workloads(w, dev, seeded, {group})
         if key not in wls:
-            sys.exit(f"bench.py --profile: unknown workload {key!r}; one of copy, " + ", ".join(
-                k for g in GROUPS for k in build_workloads(w, w.Device.planner(), lambda *a, **kw: np.zeros(a[2], dtype=kw.get("dtype", np.float32)), {g})))
+            sys.exit(f"bench.py --profile: unknown workload {key!r}; group {group!r} has: " + ", ".join(wls))
         wl = wls[key]
     us = measure_batch(w, dev, wl, launches, 10)
     scale = 1e-3 if wl.unit == "GB/s" else 1e-6
     print(json.dumps({"profile": key, "name": wl.name, "launches": launches, "us_per_step": round(us, 2),
                       "achieved": round(wl.work / us * scale, 1), "unit": wl.unit, "frac": round(wl.work / us * scale / wl.peak, 4),
                       "work_per_step": wl.work}))
+
+
+MFMA_ONLY_SRC = r"""
+// Yardstick: the MFMA work of a 256 x 256 x K tile kernel and nothing else.  Every lane takes its operand
+// fragments from A and B once (real operand data: the power the matrix cores draw depends on the bits they
+// toggle), then issues 64 v_mfma_f32_32x32x16_f16 per 64 columns of K, as the GEMM's loop does.
+typedef unsigned int u32;
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float acc16 __attribute__((ext_vector_type(16)));
+struct Args { const _Float16* a; const _Float16* b; _Float16* c; u32 m, n, k, kchunk; };
+extern "C" __global__ void __launch_bounds__(256) wkf_mfma_only(const Args g) {
+  const u32 tid = threadIdx.x;
+  h8 fa[4], fb[4];
+  for (int i = 0; i < 4; i++) fa[i] = *(const h8*)(g.a + (size_t(blockIdx.x) * 256 + tid) * 64 + i * 8);
+  for (int i = 0; i < 4; i++) fb[i] = *(const h8*)(g.b + (size_t(blockIdx.x) * 256 + tid) * 64 + i * 8);
+  acc16 acc[16];
+  for (int i = 0; i < 16; i++) acc[i] = (acc16)(0.0f);
+  for (u32 t = 0; t < g.k / 64; t++) {
+#pragma unroll
+    for (int r = 0; r < 4; r++)
+#pragma unroll
+      for (int i = 0; i < 16; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(fa[((i >> 2) + r) & 3], fb[i & 3], acc[i], 0, 0, 0);
+  }
+  float s = 0;
+  for (int i = 0; i < 16; i++) s += acc[i][0] + acc[i][7];
+  g.c[size_t(blockIdx.x) * 256 + tid] = (_Float16)s;
+}
+"""
+
+STREAM_SRC = r"""
+// Yardstick: plain streaming kernels over 1 GiB buffers (MODE 0 copy, 1 read-only, 2 write-only), U 16-byte
+// accesses per lane in flight, non-temporal bits on the loads (NTL) and the stores (NTS).
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef unsigned long long u64;
+#if NTL
+#define LD(p) __builtin_nontemporal_load(p)
+#else
+#define LD(p) (*(p))
+#endif
+#if NTS
+#define ST(p, v) __builtin_nontemporal_store(v, p)
+#else
+#define ST(p, v) (*(p) = (v))
+#endif
+extern "C" __global__ void __launch_bounds__(WG) wkf_stream(const f4* __restrict__ in, f4* __restrict__ out, u64 n4) {
+  const u64 chunk = u64(WG) * U;
+#if PERSIST
+  for (u64 base = u64(blockIdx.x) * chunk; base < n4; base += u64(gridDim.x) * chunk) {
+#else
+  { const u64 base = u64(blockIdx.x) * chunk;
+#endif
+    f4 v[U];
+#if MODE != 2
+#pragma unroll
+    for (int i = 0; i < U; i++) v[i] = LD(in + base + threadIdx.x + i * WG);
+#else
+#pragma unroll
+    for (int i = 0; i < U; i++) v[i] = (f4)(float(threadIdx.x));
+#endif
+#if MODE != 1
+#pragma unroll
+    for (int i = 0; i < U; i++) ST(out + base + threadIdx.x + i * WG, v[i]);
+#else
+    float s = 0;
+#pragma unroll
+    for (int i = 0; i < U; i++) s += v[i][0] + v[i][1] + v[i][2] + v[i][3];
+    if (s == 12345.678f) out[base + threadIdx.x][0] = s;
+#endif
+  }
+}
+"""
+
+
+def _raw_timed(lib, dev, fn, reps, warm):
+    """us per call of `fn` (which enqueues work on the library's stream): one hipEvent pair around `reps` calls."""
+    import ctypes
+    timer = ctypes.c_void_p()
+    assert lib.wkf_timer_create(dev._h, ctypes.byref(timer)) == 0
+    for _ in range(warm):
+        fn()
+    dev.sync()
+    assert lib.wkf_timer_begin(timer) == 0
+    for _ in range(reps):
+        fn()
+    assert lib.wkf_timer_end(timer) == 0
+    ns = ctypes.c_uint64()
+    assert lib.wkf_timer_elapsed_ns(timer, ctypes.byref(ns)) == 0
+    lib.wkf_timer_destroy(timer)
+    return ns.value / reps / 1e3
+
+
+def yardsticks(w, dev, seeded, which, launches):
+    """`--yardstick mfma|stream`: kernels that are not part of the library, launched through its level-0 ABI, which
+    bound what the library's kernels can reach on this machine: the matrix cores alone on the benchmark's operand
+    data (and on zeros), and plain copy / read-only / write-only streams plus the runtime's own device copy."""
+    import ctypes
+    import struct
+    from ctypes import byref, c_uint32, c_void_p
+    lib = w.load()
+
+    def dev_buf(nbytes, host=None):
+        buf = c_void_p()
+        assert lib.wkf_buffer_alloc(dev._h, nbytes, 1, byref(buf)) == 0, lib.wkf_last_error()
+        if host is not None:
+            assert lib.wkf_buffer_upload(buf, 0, host.ctypes.data_as(c_void_p), host.nbytes) == 0
+        return buf
+
+    def kernel(sig, src, entry):
+        k = c_void_p()
+        rc = lib.wkf_module_get(dev._h, sig.encode(), src.encode(), entry.encode(), byref(k))
+        assert rc == 0, lib.wkf_last_error().decode()
+        return k
+
+    out = {"yardstick": which}
+    if which == "mfma":
+        k = kernel("yardstick|mfma_only|32x32x16", MFMA_ONLY_SRC, "wkf_mfma_only")
+        rows = []
+        for label, a, b in (("config-5 operands, N(0, 0.02)", seeded(5, 0, (4096, 4096), "normal", dtype=np.float16, std=0.02),
+                             seeded(5, 1, (4096, 4096), "normal", dtype=np.float16, std=0.02)),
+                            ("zeros", np.zeros((4096, 4096), np.float16), np.zeros((4096, 4096), np.float16))):
+            ba, bb, bc = dev_buf(a.nbytes, a), dev_buf(b.nbytes, b), dev_buf(256 * 256 * 2)
+            args = struct.pack("PPPIIII", lib.wkf_buffer_ptr(ba), lib.wkf_buffer_ptr(bb), lib.wkf_buffer_ptr(bc), 4096, 4096, 4096, 0)
+            grid, block = (c_uint32 * 3)(256, 1, 1), (c_uint32 * 3)(256, 1, 1)
+            us = _raw_timed(lib, dev, lambda: lib.wkf_launch(dev._h, k, grid, block, 0, args, len(args), None), launches, 100)
+            rows.append({"data": label, "us": round(us, 2), "TFLOP/s": round(2 * 4096 ** 3 / us * 1e-6, 1),
+                         "frac_of_f16_peak": round(2 * 4096 ** 3 / us * 1e-6 / F16_MFMA_PEAK_TFLOPS, 4)})
+            for bf in (ba, bb, bc):
+                lib.wkf_buffer_release(bf)
+        out["mfma_only_4096x4096x4096_equivalent"] = rows
+    elif which == "stream":
+        n = 1 << 30
+        src_b, dst_b = dev_buf(n), dev_buf(n)
+        us = _raw_timed(lib, dev, lambda: lib.wkf_buffer_copy(dst_b, src_b, n), 10, 3)
+        rows = [{"what": "hipMemcpyAsync device to device, 1 GiB", "us": round(us, 1), "GB/s": round(2 * n / us * 1e-3)}]
+        for mode, name in ((0, "copy"), (1, "read-only"), (2, "write-only")):
+            for wg, u, persist in ((256, 4, 0), (256, 8, 0), (1024, 8, 0), (256, 8, 4)):
+                for ntl, nts in ((0, 0), (1, 1)):
+                    defs = f"#define MODE {mode}\n#define WG {wg}\n#define U {u}\n#define NTL {ntl}\n#define NTS {nts}\n#define PERSIST {1 if persist else 0}\n"
+                    k = kernel(f"yardstick|stream|{mode}|{wg}|{u}|{ntl}|{nts}|{persist}", defs + STREAM_SRC, "wkf_stream")
+                    n4 = n // 16
+                    nblk = 256 * persist if persist else n4 // (wg * u)
+                    args = struct.pack("PPQ", lib.wkf_buffer_ptr(src_b), lib.wkf_buffer_ptr(dst_b), n4)
+                    grid, block = (c_uint32 * 3)(nblk, 1, 1), (c_uint32 * 3)(wg, 1, 1)
+                    us = _raw_timed(lib, dev, lambda: lib.wkf_launch(dev._h, k, grid, block, 0, args, len(args), None), 10, 3)
+                    moved = n * (2 if mode == 0 else 1)
+                    rows.append({"what": f"{name} kernel, {wg} threads, {u} x 16 B per lane, non-temporal {'on' if ntl else 'off'}, "
+                                         + (f"{nblk} persistent blocks" if persist else "one chunk per block"),
+                                 "us": round(us, 1), "GB/s": round(moved / us * 1e-3)})
+        out["streams_1GiB"] = rows
+        for name in ("copy", "read-only", "write-only"):
+            best = max((r for r in rows if r["what"].startswith(name)), key=lambda r: r["GB/s"])
+            out["best_" + name.replace("-", "_")] = best
+    else:
+        sys.exit("bench.py --yardstick: mfma or stream")
+    print(json.dumps(out))
 
 
 def main():
@@ -421,7 +575,8 @@ def main():
                     help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
     ap.add_argument("--profile", default="", help="run one workload only (copy, c1, c2a, c2b, c3, c4_rmsnorm, c4_rope, c4_softmax, "
                                                   "c5_f32, c5_f16, c5_mlp, f16_*), for a profiler")
-    ap.add_argument("--launches", type=int, default=30, help="timed steps of --profile")
+    ap.add_argument("--launches", type=int, default=30, help="timed steps of --profile / launches of --yardstick mfma")
+    ap.add_argument("--yardstick", default="", help="mfma | stream: bounds of the machine measured with kernels outside the library")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every kernel, no collectives); --gpus must be 1.")
@@ -438,6 +593,9 @@ def main():
     props = dev.props()
     if args.profile:
         profile_one(w, dev, seeded, args.profile, args.launches)
+        return
+    if args.yardstick:
+        yardsticks(w, dev, seeded, args.yardstick, args.launches)
         return
     if args.only == "copy":
         # calibration run for the rocprofv3 counters: nothing but the 1 GiB -> 1 GiB copy kernel

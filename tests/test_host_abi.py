@@ -549,3 +549,74 @@ def test_reduce_into_plans_without_allocating_and_refuses_the_rest(wkf):
     with pytest.raises(wkf.WkfError, match="shape"):
         x.reduce_into("sum", 1, T.new(dev, np.zeros((63,), dtype=np.float32)))
     dev.close()
+
+
+def _code_object_kernels(path):
+    """The kernel records of the AMDGPU metadata note of one code object (ELF note type 32, MessagePack)."""
+    import struct
+
+    import msgpack
+    b = open(path, "rb").read()
+    assert b[:4] == b"\x7fELF"
+    shoff = struct.unpack_from("<Q", b, 0x28)[0]
+    shentsize, shnum, _ = struct.unpack_from("<HHH", b, 0x3A)
+    kernels = []
+    for i in range(shnum):
+        sh = struct.unpack_from("<IIQQQQIIQQ", b, shoff + i * shentsize)
+        if sh[1] != 7:  # SHT_NOTE
+            continue
+        p, end = sh[4], sh[4] + sh[5]
+        while p < end:
+            namesz, descsz, typ = struct.unpack_from("<III", b, p)
+            p += 12
+            name = b[p:p + namesz]
+            p += (namesz + 3) & ~3
+            desc = b[p:p + descsz]
+            p += (descsz + 3) & ~3
+            if name.startswith(b"AMDGPU") and typ == 32:
+                kernels += msgpack.unpackb(desc, raw=False)["amdhsa.kernels"]
+    return kernels
+
+
+def test_gemm_kernels_use_no_scratch_memory(tmp_path):
+    # A GEMM kernel that spills its accumulators to scratch memory still gives right results, only several times
+    # slower: every mat_mul kernel variant is compiled into an empty cache directory and the compiler's own record
+    # in each code object must show no private segment and no spilled register.
+    import glob
+    import subprocess
+    import sys
+    script = (
+        "import sys, numpy as np\n"
+        f"sys.path.insert(0, {os.path.join(ROOT, 'tests')!r})\n"
+        "from helpers import load_package\n"
+        "w = load_package(); dev = w.Device.planner(); T = w.Tensor\n"
+        "def mm(m, n, k, dt, bt=False, lead=()):\n"
+        "    a = T.new(dev, np.zeros(lead + (m, k), dtype=dt))\n"
+        "    b = T.new(dev, np.zeros(lead + ((n, k) if bt else (k, n)), dtype=dt))\n"
+        "    r = len(lead) + 2\n"
+        "    a.mat_mul(b.transpose(r - 2, r - 1) if bt else b).materialize()\n"
+        "for dt in (np.float16, np.float32):\n"
+        "    for bt in (False, True):\n"
+        "        mm(4096, 4096, 128, dt, bt)    # full 256 x 256 tiles\n"
+        "        mm(4000, 4104, 136, dt, bt)    # 256 x 256 tiles with ragged edges\n"
+        "        mm(512, 512, 256, dt, bt)      # few tiles\n"
+        "        mm(300, 264, 2048, dt, bt)     # few ragged tiles, K in slices\n"
+        "        mm(256, 256, 4096, dt, bt)     # K in slices\n"
+        "        mm(128, 384, 4096, dt, bt)     # 128 x 128 tiles (f16), K in slices\n"
+        "        mm(512, 1024, 512, dt, bt)     # 128 x 128 tiles (f16)\n"
+        "        mm(1, 1024, 512, dt, bt); mm(8, 520, 1000, dt, bt); mm(20, 264, 4096, dt, bt)  # decode sizes\n"
+        "    mm(3, 5, 7, dt)                    # the generic kernel\n"
+        "    mm(64, 64, 32, dt, lead=(3,))\n"
+    )
+    env = dict(os.environ, WKF_CACHE_DIR=str(tmp_path))
+    subprocess.run([sys.executable, "-c", script], check=True, env=env, timeout=900)
+    checked = 0
+    for path in glob.glob(os.path.join(str(tmp_path), "*.hsaco")):
+        for k in _code_object_kernels(path):
+            if not k[".name"].startswith("wkf_gemm"):
+                continue
+            checked += 1
+            assert k[".private_segment_fixed_size"] == 0 and not k[".uses_dynamic_stack"], (k[".name"], k[".private_segment_fixed_size"])
+            assert k[".vgpr_spill_count"] == 0 and k[".sgpr_spill_count"] == 0, (k[".name"], k[".vgpr_spill_count"], k[".sgpr_spill_count"])
+            assert k[".vgpr_count"] <= 512
+    assert checked >= 22, f"only {checked} GEMM kernels were compiled: the shapes above no longer reach the variants"
