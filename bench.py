@@ -272,6 +272,14 @@ def build_workloads(w, dev, seeded, which, with_cpu=False):
         del hbm
         out["c5_mlp"] = Workload("config5c: GEMM f16 [2048x4096]x[4096x11008]", [[am.mat_mul(bm)]], 184683593728, "TFLOP/s",
                                  F16_MFMA_PEAK_TFLOPS, "f16", cpu=mlp_cpu)
+    if "long" in which:
+        # rows longer than a block's registers (no BASELINE configuration; the reference's reduce takes any length)
+        xs = [T.new(dev, seeded(4, 40 + r, (256, 262144), "normal")) for r in range(2)]
+        out["long_softmax"] = Workload("long rows: softmax f32 [256,262144]", [[x.softmax_last_dim()] for x in xs], 2 * 256 * 262144 * 4,
+                                       "GB/s", HBM_PEAK_GBS)
+        xf = [T.new(dev, seeded(4, 44 + r, (64, 262144), "normal")) for r in range(2)]
+        out["long_softmax_few"] = Workload("few long rows: softmax f32 [64,262144]", [[x.softmax_last_dim()] for x in xf],
+                                           2 * 64 * 262144 * 4, "GB/s", HBM_PEAK_GBS)
     if "f16" in which:
         # the f16 forms of the memory-bound kernels (no BASELINE configuration names them; no CPU figure)
         F16 = np.float16
@@ -361,7 +369,7 @@ def cpu_baseline(wl):
                       "oracle/port.c with OpenMP"}
 
 
-GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16")
+GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16", "long")
 
 
 def plan_only(w):
@@ -436,8 +444,9 @@ extern "C" __global__ void __launch_bounds__(256) wkf_mfma_only(const Args g) {
 """
 
 STREAM_SRC = r"""
-// Yardstick: plain streaming kernels over 1 GiB buffers (MODE 0 copy, 1 read-only, 2 write-only), U 16-byte
-// accesses per lane in flight, non-temporal bits on the loads (NTL) and the stores (NTS).
+// Yardstick: plain streaming kernels over 1 GiB buffers (MODE 0 copy, 1 read-only, 2 write-only, 3 two reads and
+// one write: out = in + in2), U 16-byte accesses per lane and stream in flight, non-temporal bits on the loads
+// (NTL) and the stores (NTS).
 typedef float f4 __attribute__((ext_vector_type(4)));
 typedef unsigned long long u64;
 #if NTL
@@ -450,7 +459,7 @@ typedef unsigned long long u64;
 #else
 #define ST(p, v) (*(p) = (v))
 #endif
-extern "C" __global__ void __launch_bounds__(WG) wkf_stream(const f4* __restrict__ in, f4* __restrict__ out, u64 n4) {
+extern "C" __global__ void __launch_bounds__(WG) wkf_stream(const f4* __restrict__ in, f4* __restrict__ out, u64 n4, const f4* __restrict__ in2) {
   const u64 chunk = u64(WG) * U;
 #if PERSIST
   for (u64 base = u64(blockIdx.x) * chunk; base < n4; base += u64(gridDim.x) * chunk) {
@@ -458,7 +467,15 @@ extern "C" __global__ void __launch_bounds__(WG) wkf_stream(const f4* __restrict
   { const u64 base = u64(blockIdx.x) * chunk;
 #endif
     f4 v[U];
-#if MODE != 2
+#if MODE == 3
+    f4 v2[U];
+#pragma unroll
+    for (int i = 0; i < U; i++) v[i] = LD(in + base + threadIdx.x + i * WG);
+#pragma unroll
+    for (int i = 0; i < U; i++) v2[i] = LD(in2 + base + threadIdx.x + i * WG);
+#pragma unroll
+    for (int i = 0; i < U; i++) v[i] += v2[i];
+#elif MODE != 2
 #pragma unroll
     for (int i = 0; i < U; i++) v[i] = LD(in + base + threadIdx.x + i * WG);
 #else
@@ -537,27 +554,33 @@ def yardsticks(w, dev, seeded, which, launches):
         out["mfma_only_4096x4096x4096_equivalent"] = rows
     elif which == "stream":
         n = 1 << 30
-        src_b, dst_b = dev_buf(n), dev_buf(n)
+        src_b, dst_b, src2_b = dev_buf(n), dev_buf(n), dev_buf(n)
         us = _raw_timed(lib, dev, lambda: lib.wkf_buffer_copy(dst_b, src_b, n), 10, 3)
         rows = [{"what": "hipMemcpyAsync device to device, 1 GiB", "us": round(us, 1), "GB/s": round(2 * n / us * 1e-3)}]
-        for mode, name in ((0, "copy"), (1, "read-only"), (2, "write-only")):
+        # the cost of a launch itself: the read-only kernel over 4 KiB (one block), back to back on the stream
+        k0 = kernel("yardstick|stream|1|256|1|0|0|0", "#define MODE 1\n#define WG 256\n#define U 1\n#define NTL 0\n#define NTS 0\n#define PERSIST 0\n" + STREAM_SRC, "wkf_stream")
+        args0 = struct.pack("PPQP", lib.wkf_buffer_ptr(src_b), lib.wkf_buffer_ptr(dst_b), 256, lib.wkf_buffer_ptr(src2_b))
+        g0, b0 = (c_uint32 * 3)(1, 1, 1), (c_uint32 * 3)(256, 1, 1)
+        us = _raw_timed(lib, dev, lambda: lib.wkf_launch(dev._h, k0, g0, b0, 0, args0, len(args0), None), 500, 50)
+        out["launch_floor_us"] = round(us, 2)
+        for mode, name in ((0, "copy"), (1, "read-only"), (2, "write-only"), (3, "two reads + one write")):
             for wg, u, persist in ((256, 4, 0), (256, 8, 0), (1024, 8, 0), (256, 8, 4)):
                 for ntl, nts in ((0, 0), (1, 1)):
                     defs = f"#define MODE {mode}\n#define WG {wg}\n#define U {u}\n#define NTL {ntl}\n#define NTS {nts}\n#define PERSIST {1 if persist else 0}\n"
                     k = kernel(f"yardstick|stream|{mode}|{wg}|{u}|{ntl}|{nts}|{persist}", defs + STREAM_SRC, "wkf_stream")
                     n4 = n // 16
                     nblk = 256 * persist if persist else n4 // (wg * u)
-                    args = struct.pack("PPQ", lib.wkf_buffer_ptr(src_b), lib.wkf_buffer_ptr(dst_b), n4)
+                    args = struct.pack("PPQP", lib.wkf_buffer_ptr(src_b), lib.wkf_buffer_ptr(dst_b), n4, lib.wkf_buffer_ptr(src2_b))
                     grid, block = (c_uint32 * 3)(nblk, 1, 1), (c_uint32 * 3)(wg, 1, 1)
                     us = _raw_timed(lib, dev, lambda: lib.wkf_launch(dev._h, k, grid, block, 0, args, len(args), None), 10, 3)
-                    moved = n * (2 if mode == 0 else 1)
+                    moved = n * {0: 2, 1: 1, 2: 1, 3: 3}[mode]
                     rows.append({"what": f"{name} kernel, {wg} threads, {u} x 16 B per lane, non-temporal {'on' if ntl else 'off'}, "
                                          + (f"{nblk} persistent blocks" if persist else "one chunk per block"),
                                  "us": round(us, 1), "GB/s": round(moved / us * 1e-3)})
         out["streams_1GiB"] = rows
-        for name in ("copy", "read-only", "write-only"):
+        for name in ("copy", "read-only", "write-only", "two reads + one write"):
             best = max((r for r in rows if r["what"].startswith(name)), key=lambda r: r["GB/s"])
-            out["best_" + name.replace("-", "_")] = best
+            out["best_" + name.replace("-", "_").replace(" + ", "_").replace(" ", "_")] = best
     else:
         sys.exit("bench.py --yardstick: mfma or stream")
     print(json.dumps(out))
@@ -570,7 +593,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="only the headline configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
-    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16 for the detail table")
+    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16,long for the detail table")
     ap.add_argument("--plan-only", action="store_true",
                     help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
     ap.add_argument("--profile", default="", help="run one workload only (copy, c1, c2a, c2b, c3, c4_rmsnorm, c4_rope, c4_softmax, "

@@ -530,6 +530,54 @@ def test_row_kernels_on_rows_that_do_not_split_evenly(gpu, rows, n, dtype):
     assert np.allclose(got[2].astype(np.float64), total, rtol=1e-5 if dtype == np.float32 else 4e-3)
 
 
+LONG_ROWS = [(128, 100003, np.float32), (130, 262144, np.float32), (129, 70000, np.float32), (128, 140002, np.float16),
+             (131, 131080, np.float16)]
+
+
+@pytest.mark.parametrize("rows,n,dtype", LONG_ROWS, ids=[f"{r}x{n}_{np.dtype(d).name}" for r, n, d in LONG_ROWS])
+def test_rows_longer_than_a_blocks_registers_stay_one_kernel(gpu, rows, n, dtype):
+    # Rows beyond 65536 floats do not fit the registers of a block: with enough rows to occupy the chip one block
+    # per row streams its row once per stage and once more for the result, in ONE launch (the reference's reduce
+    # takes any length in one kernel, src/reduce.rs:340-350); odd lengths take narrower vectors.
+    x = data((rows, n), -3, 3, dtype, rows * 11 + n)
+    w = data((n,), 0.5, 1.5, dtype, n + 1)
+    api = HipAPI(gpu)
+    tx, tw = api.tensor(x), api.tensor(w)
+    ox, ow = OTensor(x), OTensor(w)
+    progs = [tx.softmax_last_dim()]
+    want = [ox.softmax_last_dim().to_numpy()]
+    if dtype == np.float32:
+        progs.append(tx.layer_norm(tw, 1e-5))
+        want.append(ox.layer_norm(ow, 1e-5).to_numpy())
+    got = hip_values_many(progs)
+    for p in progs:
+        assert [k.kind for k in p.kernels()] == ["row"] and "streamed" in p.kernels()[0].detail, [k.detail for k in p.kernels()]
+    rtol = 1e-5 if dtype == np.float32 else 2e-3
+    for i in range(len(got)):
+        assert got[i].shape == want[i].shape
+        assert np.allclose(got[i].astype(np.float64), want[i].astype(np.float64), rtol=rtol, atol=1e-9 if dtype == np.float32 else 1e-7), i
+    assert np.allclose(got[0].astype(np.float64).sum(1), 1.0, atol=1e-5 if dtype == np.float32 else 5e-2)
+    assert np.array_equal(np.argmax(got[0], 1), np.argmax(x, 1))
+    # both reductions of the rows in one pass (materialize_many): also one streamed kernel, the same values as alone
+    if dtype == np.float32:
+        pair = [tx.max(1), (tx.clone() - 1.0).exp().sum(1)]
+        m, se = hip_values_many(pair)
+        assert np.array_equal(m, x.max(1))
+        ref = np.exp((x - np.float32(1.0)).astype(np.float64)).astype(np.float32).astype(np.float64).sum(1)
+        assert np.allclose(se, ref, rtol=1e-5)
+
+
+def test_few_long_rows_fold_across_the_grid(gpu):
+    # with only a few rows a block per row would leave most compute units idle: those keep the reductions that are
+    # folded across the whole grid (several launches), with the same values
+    x = data((5, 100003), -3, 3, np.float32, 77)
+    api = HipAPI(gpu)
+    t = api.tensor(x).softmax_last_dim()
+    got = hip_values(t)
+    assert len(t.kernels()) > 1
+    assert np.allclose(got, OTensor(x).softmax_last_dim().to_numpy(), rtol=1e-5, atol=1e-9)
+
+
 # ---- the benchmark configurations at full size ------------------------------------------------------------------------------
 
 def test_config1_fused_unary_chain_full_size(gpu):

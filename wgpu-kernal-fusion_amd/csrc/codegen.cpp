@@ -823,6 +823,7 @@ std::string row_signature(const RowSpec& s) {
   if (s.store_scalars) o << "|scalars";
   else o << "|final{" << s.final.signature() << "}";
   if (s.ragged) o << "|ragged";
+  if (s.streamed) o << "|streamed";
   return o.str();
 }
 
@@ -857,7 +858,7 @@ std::string row_source(const RowSpec& s) {
     if (round_h) o << kRoundH;
   }
   o << kRowHelpers;
-  o << "struct Args { void* p[" << K + NOUT << "]; u32 nrows; " << (s.ragged ? "u32 nvec; " : "") << "u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
+  o << "struct Args { void* p[" << K + NOUT << "]; u32 nrows; " << (s.ragged || s.streamed ? "u32 nvec; " : "") << "u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
     << "]; u32 ostride[" << K + NOUT << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
   // operand types as every program sees them: the K full operands, then one scalar per earlier stage
   std::vector<DType> types;
@@ -888,6 +889,88 @@ std::string row_source(const RowSpec& s) {
     for (int d = 0; d < Ro; d++) e << " + i" << d << " * a.ostride[" << k << "][" << d << "]";
     return e.str();
   };
+  if (s.streamed) {
+    // ---- rows longer than the registers of a block: one pass over the row per stage, one more for the result ----
+    const int U = NV;
+    for (int k = 0; k < K; k++) {
+      const char* ct = ctype(s.in[k].dtype);
+      o << "  const " << ct << "* q" << k << " = ((const " << ct << "*)a.p[" << k << "]) + (" << base_expr(k) << ");\n";
+      if (s.in[k].axis_stride == 0) o << "  const " << ct << " s" << k << " = q" << k << "[0];\n";
+    }
+    auto sargs = [&](int u, int e, int nscalars) {
+      std::ostringstream c;
+      for (int k = 0; k < K; k++) {
+        if (s.in[k].axis_stride == 0) c << "s" << k;
+        else {
+          c << "x" << k << "_" << u;
+          if (V > 1) c << "[" << e << "]";
+        }
+        c << ", ";
+      }
+      for (int q = 0; q < nscalars; q++) c << "r" << q << ", ";
+      return c.str();
+    };
+    // `last`: the final pass streams (nothing reads the row again); earlier passes leave it in the caches
+    auto emit_loads = [&](bool last) {
+      for (int u = 0; u < U; u++) o << "    const u32 j" << u << " = base + t + " << u * T << "u; const bool ok" << u << " = j" << u << " < a.nvec;\n";
+      for (int k = 0; k < K; k++) {
+        if (s.in[k].axis_stride == 0) continue;
+        std::string vt = vtype(s.in[k].dtype, V);
+        for (int u = 0; u < U; u++) {
+          o << "    const " << vt << " x" << k << "_" << u << " = !ok" << u << " ? (" << vt << ")(0) : ";
+          if (last) o << "__builtin_nontemporal_load((const " << vt << "*)(q" << k << " + j" << u << " * " << V << "u));\n";
+          else o << "*(const " << vt << "*)(q" << k << " + j" << u << " * " << V << "u);\n";
+        }
+      }
+    };
+    const bool last_is_stage = s.store_scalars;
+    for (int k = 0; k < S; k++) {
+      const RowStage& st = s.stages[k];
+      o << "  float acc" << k << " = " << seed_text(st.rop) << ";\n";
+      o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(st.rop) << "; };\n";
+      o << "  for (u32 base = 0; base < a.nvec; base += " << T * U << "u) {\n";
+      emit_loads(last_is_stage && k == S - 1);
+      for (int u = 0; u < U; u++) {
+        o << "    if (ok" << u << ") {\n";
+        for (int e = 0; e < V; e++)
+          o << "      acc" << k << " = fold" << k << "((float)wkf_pre" << k << "(" << sargs(u, e, k) << "a.c + " << pre_off[k] << "), acc" << k << ");\n";
+        o << "    }\n";
+      }
+      o << "  }\n";
+      o << "  acc" << k << " = wkf_lanes_fold_with<64>(acc" << k << ", fold" << k << ");\n";
+      o << "  if ((threadIdx.x & 63u) == 0u) wkf_partial[" << k << "][threadIdx.x >> 6] = acc" << k << ";\n";
+      o << "  __syncthreads();\n";
+      o << "  acc" << k << " = wkf_partial[" << k << "][0];\n";
+      o << "  for (u32 w = 1; w < " << T / 64 << "u; w++) acc" << k << " = fold" << k << "(wkf_partial[" << k << "][w], acc" << k << ");\n";
+      o << "  const " << ctype(st.post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(st.pre.result_dtype()) << ")acc" << k
+        << ", a.c + " << post_off[k] << ");\n";
+    }
+    if (s.store_scalars) {
+      o << "  if (live && t == 0u) {\n";
+      for (int k = 0; k < S; k++) {
+        const char* st = ctype(s.stages[k].post.result_dtype());
+        o << "    ((" << st << "*)a.p[" << K + k << "])[" << base_expr(K + k) << "] = r" << k << ";\n";
+      }
+      o << "  }\n}\n";
+      return o.str();
+    }
+    const char* sot = ctype(s.out_dtype);
+    std::string ovt = vtype(s.out_dtype, V);
+    o << "  " << sot << "* qo = ((" << sot << "*)a.p[" << K << "]) + (" << base_expr(K) << ");\n";
+    o << "  for (u32 base = 0; base < a.nvec; base += " << T * U << "u) {\n";
+    emit_loads(true);
+    for (int u = 0; u < U; u++) {
+      o << "    if (live && ok" << u << ") {\n      " << ovt << " ov;\n";
+      for (int e = 0; e < V; e++) {
+        o << "      ov";
+        if (V > 1) o << "[" << e << "]";
+        o << " = wkf_final(" << sargs(u, e, S) << "a.c + " << final_off << ");\n";
+      }
+      o << "      __builtin_nontemporal_store(ov, (" << ovt << "*)(qo + j" << u << " * " << V << "u));\n    }\n";
+    }
+    o << "  }\n}\n";
+    return o.str();
+  }
   // the row of every operand comes into registers once
   for (int k = 0; k < K; k++) {
     const char* ct = ctype(s.in[k].dtype);
@@ -976,7 +1059,7 @@ std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a) {
   std::vector<unsigned char> b;
   for (void* p : a.ptrs) putp(b, p);
   put32(b, a.nrows);
-  if (s.ragged) put32(b, a.nvec);
+  if (s.ragged || s.streamed) put32(b, a.nvec);
   for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? a.oshape[d] : 1);
   for (uint32_t v : a.offsets) put32(b, v);
   for (const auto& st : a.ostrides) {

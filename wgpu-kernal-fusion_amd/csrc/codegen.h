@@ -141,6 +141,10 @@ struct RowSpec {
   // ragged: the row holds `nvec` vectors (a launch argument) with (NV - 1) * T < nvec <= NV * T; lanes whose last
   // vector lies past the end of the row neither load, fold nor store it
   bool ragged = false;
+  // streamed: the row is longer than a block's registers hold.  One block of T lanes per row walks the row's `nvec`
+  // vectors (a launch argument) once per stage and once more for the final expression, `vectors_per_lane` vectors
+  // of every operand in flight per lane; the passes after the first find the row in the caches when it fits them.
+  bool streamed = false;
   std::vector<ReduceOperandSpec> in;    // axis_stride 1 (row in registers) or 0 (one scalar per row)
   std::vector<RowStage> stages;
   Program final;                        // same operand numbering as a stage's pre

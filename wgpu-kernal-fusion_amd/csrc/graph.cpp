@@ -693,11 +693,22 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
     T = T_wide;
     ragged = true;
   }
-  const size_t NV = (nvec + T - 1) / T;
-  if (NV > max_nv || NV * V * K > 128) return false;
+  size_t NV = (nvec + T - 1) / T;
   size_t nrows = 1;
   for (size_t d : out_shape) nrows *= d;
   if (nrows > 0xffffffffull) return false;
+  bool streamed = false;
+  if (NV > max_nv || NV * V * K > 128) {
+    // The row does not fit the registers of a block.  With enough rows to occupy the chip, one block per row
+    // streams its row once per stage and once more for the result, in ONE launch; the passes after the first
+    // find the row in the caches when it fits them.  With only a few rows a block per row would leave most
+    // compute units idle: the caller then folds each reduction across the whole grid instead (several launches).
+    if (nrows < st_.row_stream_min_rows || nvec < 1024) return false;
+    streamed = true;
+    ragged = false;
+    T = 1024;
+    NV = std::max<size_t>(1, std::min<size_t>(4, 8 / std::max<size_t>(1, K)));  // vectors in flight per lane and operand
+  }
 
   // operand numbering: full operands 0..K-1, then the scalars
   auto renumber = [&](Program& p) {
@@ -712,6 +723,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   spec.block = std::max(256, T);
   spec.vectors_per_lane = int(NV);
   spec.ragged = ragged;
+  spec.streamed = streamed;
   spec.stages = rb.stages;
   spec.final = final;
   spec.store_scalars = scalars;
@@ -754,6 +766,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
     << rb.stages.size() << " operands=" << K + NOUT;
   if (scalars) d << " reductions=" << S;
   if (ragged) d << " ragged";
+  if (streamed) d << " streamed";
   r.detail = d.str();
   record(std::move(r), k, row_pack_args(spec, args));
   return true;
