@@ -400,7 +400,7 @@ def plan_only(w):
 def profile_one(w, dev, seeded, key, launches):
     """`--profile KEY`: nothing but `launches` steps of one workload (after 10 untimed ones), for a profiler run
     (rocprofv3 --kernel-trace --stats / --pmc ... -- python3 bench.py --profile KEY)."""
-    group = key.split("_")[0]
+    group = next((g for g in GROUPS if key.startswith(g)), key)
     if key == "copy":
         x = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32))
         wl = Workload("copy 1 GiB -> 1 GiB", [[x.resize([1 << 28])]], 2 * (1 << 30), "GB/s", HBM_PEAK_GBS)
