@@ -397,9 +397,10 @@ def plan_only(w):
                       "kernels_from_disk_cache": after["disk_hits"] - before["disk_hits"]}))
 
 
-def profile_one(w, dev, seeded, key, launches):
-    """`--profile KEY`: nothing but `launches` steps of one workload (after 10 untimed ones), for a profiler run
-    (rocprofv3 --kernel-trace --stats / --pmc ... -- python3 bench.py --profile KEY)."""
+def profile_one(w, dev, seeded, key, launches, warm_ms):
+    """`--profile KEY`: nothing but `launches` steps of one workload, for a profiler run (rocprofv3 --kernel-trace
+    --stats / --pmc ... -- python3 bench.py --profile KEY).  Before them, untimed steps for `warm_ms` milliseconds (at
+    least 10 steps): after an idle spell the GPU takes tens of milliseconds to reach its working clocks."""
     group = next((g for g in GROUPS if key.startswith(g)), key)
     if key == "copy":
         x = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32))
@@ -409,9 +410,18 @@ def profile_one(w, dev, seeded, key, launches):
         if key not in wls:
             sys.exit(f"bench.py --profile: unknown workload {key!r}; group {group!r} has: " + ", ".join(wls))
         wl = wls[key]
+    dev.set_timing(False)
+    t_end = time.perf_counter() + warm_ms * 1e-3
+    i = 0
+    while time.perf_counter() < t_end:
+        wl.step(i)
+        i += 1
+        if i % 50 == 0:
+            dev.sync()
+    dev.sync()
     us = measure_batch(w, dev, wl, launches, 10)
     scale = 1e-3 if wl.unit == "GB/s" else 1e-6
-    print(json.dumps({"profile": key, "name": wl.name, "launches": launches, "us_per_step": round(us, 2),
+    print(json.dumps({"profile": key, "warm_steps": i + 10, "name": wl.name, "launches": launches, "us_per_step": round(us, 2),
                       "achieved": round(wl.work / us * scale, 1), "unit": wl.unit, "frac": round(wl.work / us * scale / wl.peak, 4),
                       "work_per_step": wl.work}))
 
@@ -599,6 +609,7 @@ def main():
     ap.add_argument("--profile", default="", help="run one workload only (copy, c1, c2a, c2b, c3, c4_rmsnorm, c4_rope, c4_softmax, "
                                                   "c5_f32, c5_f16, c5_mlp, f16_*), for a profiler")
     ap.add_argument("--launches", type=int, default=30, help="timed steps of --profile / launches of --yardstick mfma")
+    ap.add_argument("--warm-ms", type=float, default=300.0, help="--profile: milliseconds of untimed steps before the timed ones")
     ap.add_argument("--yardstick", default="", help="mfma | stream: bounds of the machine measured with kernels outside the library")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -615,7 +626,7 @@ def main():
     dev = w.Device.new(0)
     props = dev.props()
     if args.profile:
-        profile_one(w, dev, seeded, args.profile, args.launches)
+        profile_one(w, dev, seeded, args.profile, args.launches, args.warm_ms)
         return
     if args.yardstick:
         yardsticks(w, dev, seeded, args.yardstick, args.launches)

@@ -99,6 +99,19 @@ def test_interior_exp_on_f16_is_correctly_rounded_for_every_argument(gpu):
     assert_ulp(got, want, 0, "silu on f16")
 
 
+@pytest.mark.parametrize("op", sorted(TRANS_UNARY), ids=str)
+def test_interior_transcendentals_on_f16_are_correctly_rounded_for_every_argument(gpu, op):
+    # a transcendental op that feeds further arithmetic on an f16 tensor must be the correctly rounded f16 value: the
+    # f32 library decides it for most arguments and the f64 routine for the rest; all 63488 finite f16 values
+    # (outside the function's domain both sides give NaN)
+    bits = np.arange(0, 1 << 16, dtype=np.uint16)
+    x = bits.view(np.float16)
+    x = x[np.isfinite(x)]
+    with np.errstate(all="ignore"):
+        got, want = both(gpu, lambda t: getattr(t, op)() * 1.0, x)
+    assert_ulp(got, want, 0, f"{op} on f16")
+
+
 def test_trig_far_arguments_take_the_slow_path(gpu):
     x = np.array([0.0, 1.0, 99999.0, 100001.0, 1e7, -3e9, 1e30, np.inf, np.nan, -0.0] * 13, dtype=np.float32)
     got, want = both(gpu, lambda t: (t.sin() * 2.0) + t.cos() * 0.5, x)
@@ -682,7 +695,9 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                # 5 to 32 rows against a row-major B: the MFMA decode kernel (LDS transpose reads), K in slices
                (32, 4096, 512), (17, 264, 1000), (8, 1000, 4096), (31, 72, 2048), (5, 4104, 136), (24, 8, 8200), (32, 1028, 700),
                # 128 x 128 tiles (products that would not fill the chip with 256 x 256 ones): full, ragged, K in slices
-               (128, 128, 64), (129, 136, 64), (384, 640, 192), (200, 1000, 520), (511, 136, 2048), (33, 4096, 1024)]
+               (128, 128, 64), (129, 136, 64), (384, 640, 192), (200, 1000, 520), (511, 136, 2048), (33, 4096, 1024),
+               # full tiles that leave a partly filled last round on 256 compute units (272, 300 and 257 tiles)
+               (4096, 4352, 512), (2560, 7680, 1024), (256, 65792, 2048)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -698,7 +713,8 @@ def test_mat_mul(gpu, m, n, k, dtype, tol):
 
 
 BT_SHAPES = [(256, 512, 128), (300, 264, 2048), (100, 136, 72), (513, 260, 328), (1, 1024, 512), (7, 520, 1000),
-             (32, 264, 4096), (2, 4100, 96), (20, 100, 64), (3, 5, 7), (33, 2048, 1024), (300, 1000, 515)]
+             (32, 264, 4096), (2, 4100, 96), (20, 100, 64), (3, 5, 7), (33, 2048, 1024), (300, 1000, 515),
+             (4096, 4352, 512)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -786,5 +802,9 @@ def test_config5_gemm_full_size(gpu, name, m, n, k, dtype, tol):
     a = seeded(5, 0, (m, k), "normal", dtype=dtype, std=0.02)
     b = seeded(5, 1, (k, n), "normal", dtype=dtype, std=0.02)
     api = HipAPI(gpu)
-    got = hip_values(api.tensor(a).mat_mul(api.tensor(b)))
+    prod = api.tensor(a).mat_mul(api.tensor(b))
+    got = hip_values(prod)
     gemm_check(got, a, b, tol)
+    # the same product twice gives the same bits
+    again = hip_values(api.tensor(a).mat_mul(api.tensor(b)))
+    assert np.array_equal(got, again)

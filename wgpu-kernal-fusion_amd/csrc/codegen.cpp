@@ -41,10 +41,16 @@ bool uses_math(const Program& p, MathPolicy policy) {
   return false;
 }
 
+// An exact transcendental op with an f16 result outside exact-math mode: the f32 library settles the f16 rounding
+// for all but a few arguments in a thousand, and only those go through f64 (wkf_h_via_f32 below).
+bool h_via_f32(const Program& p, size_t i, MathPolicy policy) {
+  return p.ins[i].dtype == DType::F16 && policy != MathPolicy::Exact && exact_op(p, i, policy);
+}
+
 // Uses the branch-free sin / cos core, i.e. needs the `far` flag and a far variant.
 bool uses_trig(const Program& p, MathPolicy policy) {
   for (size_t i = 0; i < p.ins.size(); i++)
-    if ((p.ins[i].op == Op::Sin || p.ins[i].op == Op::Cos) && exact_op(p, i, policy)) return true;
+    if ((p.ins[i].op == Op::Sin || p.ins[i].op == Op::Cos) && exact_op(p, i, policy) && !h_via_f32(p, i, policy)) return true;
   return false;
 }
 
@@ -58,6 +64,15 @@ const char* const kRoundH =
     "  const _Float16 lo = (_Float16)(y * 0x1.fffffep-1f), hi = (_Float16)(y * 0x1.000002p+0f);\n"
     "  if (__builtin_expect(lo == hi, 1)) return lo;\n"
     "  return (_Float16)d;\n"
+    "}\n"
+    // An f16 result that feeds further arithmetic must be the correctly rounded one.  The f32 library's value y is
+    // within a few f32 ulps of the true one; y (1 -+ 2^-20) brackets it with room to spare (16 ulps), and when both
+    // ends round to the same f16 value that value is the answer.  Otherwise (about two arguments in a thousand) the
+    // f64 routine decides.  Conversions are compared, not bits, so zeros, subnormals, infinities and NaN need no case.
+    "template <typename F> static __device__ __forceinline__ _Float16 wkf_h_via_f32(float y, F exact) {\n"
+    "  const _Float16 lo = (_Float16)(y * 0x1.ffffe0p-1f), hi = (_Float16)(y * 0x1.000010p+0f);\n"
+    "  if (__builtin_expect(lo == hi, 1)) return lo;\n"
+    "  return exact();\n"
     "}\n";
 
 bool is_transcendental(Op o) {
@@ -178,6 +193,12 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
           // f16 result: 2^(x log2 e) on the hardware unit (relative error about 2^-21 for any f16 argument,
           // a thousand times finer than the f16 grid); the f32 library's exp would cost more than the loads.
           o << "(_Float16)__builtin_amdgcn_exp2f((float)" << a << " * 0x1.715476p+0f)";
+          break;
+        }
+        if (h && exact && policy != MathPolicy::Exact && in.op != Op::Sqrt) {
+          // an interior transcendental on f16: the f32 library, and the library's f64 routine where that cannot decide
+          const std::string f = lib_fn(in.op);
+          o << "wkf_h_via_f32(" << f << "f((float)" << a << "), [&] { return wkf_round_h(" << f << "((double)" << a << ")); })";
           break;
         }
         std::string call = math_call(in.op, h ? "(float)" + a : a, exact, far_variant, h);
