@@ -845,6 +845,7 @@ std::string row_signature(const RowSpec& s) {
   else o << "|final{" << s.final.signature() << "}";
   if (s.ragged) o << "|ragged";
   if (s.streamed) o << "|streamed";
+  if (s.online_max_sum) o << "|online";
   return o.str();
 }
 
@@ -945,7 +946,41 @@ std::string row_source(const RowSpec& s) {
       }
     };
     const bool last_is_stage = s.store_scalars;
-    for (int k = 0; k < S; k++) {
+    auto block_fold = [&](int k) {  // acc<k> of every lane -> the row's value in every lane
+      o << "  acc" << k << " = wkf_lanes_fold_with<64>(acc" << k << ", fold" << k << ");\n";
+      o << "  if ((threadIdx.x & 63u) == 0u) wkf_partial[" << k << "][threadIdx.x >> 6] = acc" << k << ";\n";
+      o << "  __syncthreads();\n";
+      o << "  acc" << k << " = wkf_partial[" << k << "][0];\n";
+      o << "  for (u32 w = 1; w < " << T / 64 << "u; w++) acc" << k << " = fold" << k << "(wkf_partial[" << k << "][w], acc" << k << ");\n";
+    };
+    if (s.online_max_sum) {
+      // stages 0 and 1 in one pass: every lane keeps a running maximum m and the sum of exp(x - m) over what it
+      // has seen; when m grows the sum is rescaled by exp(old m - new m).  Lanes are combined the same way.
+      const char* mt = ctype(s.stages[0].post.result_dtype());
+      o << "  float acc0 = " << seed_text(ReduceOp::Max) << ", acc1 = 0.0f;\n";
+      o << "  auto fold0 = [](float v, float a) { return fmaxf(v, a); };\n";
+      o << "  auto fold1 = [](float v, float a) { return v + a; };\n";
+      o << "  for (u32 base = 0; base < a.nvec; base += " << T * U << "u) {\n";
+      emit_loads(last_is_stage && S == 2);
+      for (int u = 0; u < U; u++) {
+        o << "    if (ok" << u << ") {\n";
+        o << "      float cm = acc0;\n";
+        for (int e = 0; e < V; e++) o << "      cm = fmaxf((float)wkf_pre0(" << sargs(u, e, 0) << "a.c + " << pre_off[0] << "), cm);\n";
+        o << "      acc1 *= expf(acc0 - cm);\n      acc0 = cm;\n";
+        o << "      const " << mt << " r0 = wkf_post0((" << ctype(s.stages[0].pre.result_dtype()) << ")cm, a.c + " << post_off[0] << ");\n";
+        for (int e = 0; e < V; e++) o << "      acc1 += (float)wkf_pre1(" << sargs(u, e, 1) << "a.c + " << pre_off[1] << ");\n";
+        o << "    }\n";
+      }
+      o << "  }\n";
+      o << "  const float lane_max = acc0;\n";
+      block_fold(0);
+      o << "  acc1 *= expf(lane_max - acc0);\n";
+      block_fold(1);
+      for (int k = 0; k < 2; k++)
+        o << "  const " << ctype(s.stages[k].post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(s.stages[k].pre.result_dtype())
+          << ")acc" << k << ", a.c + " << post_off[k] << ");\n";
+    }
+    for (int k = s.online_max_sum ? 2 : 0; k < S; k++) {
       const RowStage& st = s.stages[k];
       o << "  float acc" << k << " = " << seed_text(st.rop) << ";\n";
       o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(st.rop) << "; };\n";
@@ -958,11 +993,7 @@ std::string row_source(const RowSpec& s) {
         o << "    }\n";
       }
       o << "  }\n";
-      o << "  acc" << k << " = wkf_lanes_fold_with<64>(acc" << k << ", fold" << k << ");\n";
-      o << "  if ((threadIdx.x & 63u) == 0u) wkf_partial[" << k << "][threadIdx.x >> 6] = acc" << k << ";\n";
-      o << "  __syncthreads();\n";
-      o << "  acc" << k << " = wkf_partial[" << k << "][0];\n";
-      o << "  for (u32 w = 1; w < " << T / 64 << "u; w++) acc" << k << " = fold" << k << "(wkf_partial[" << k << "][w], acc" << k << ");\n";
+      block_fold(k);
       o << "  const " << ctype(st.post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(st.pre.result_dtype()) << ")acc" << k
         << ", a.c + " << post_off[k] << ");\n";
     }

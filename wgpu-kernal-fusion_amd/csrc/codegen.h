@@ -145,6 +145,10 @@ struct RowSpec {
   // vectors (a launch argument) once per stage and once more for the final expression, `vectors_per_lane` vectors
   // of every operand in flight per lane; the passes after the first find the row in the caches when it fits them.
   bool streamed = false;
+  // streamed rows whose first two stages are max(x) and sum(exp(x - max)) (softmax): both are folded in ONE pass
+  // with a running maximum (the running sum is rescaled by exp(old max - new max) whenever the maximum grows), so
+  // the row is read twice in all instead of three times
+  bool online_max_sum = false;
   std::vector<ReduceOperandSpec> in;    // axis_stride 1 (row in registers) or 0 (one scalar per row)
   std::vector<RowStage> stages;
   Program final;                        // same operand numbering as a stage's pre

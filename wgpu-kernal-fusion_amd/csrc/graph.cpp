@@ -725,6 +725,21 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   spec.ragged = ragged;
   spec.streamed = streamed;
   spec.stages = rb.stages;
+  if (streamed && rb.stages.size() >= 2) {
+    // softmax's pair of stages, max(x) then sum(exp(x - max)), is folded in one pass over a streamed row
+    const RowStage& s0 = rb.stages[0];
+    const RowStage& s1 = rb.stages[1];
+    auto is_load = [](const Instr& in, int operand) { return in.op == Op::Load && in.operand == operand; };
+    const bool max_of_x = s0.rop == ReduceOp::Max && s0.pre.ins.size() == 1 && is_load(s0.pre.ins[0], 0) && s0.post.ins.size() == 1;
+    bool sum_exp = s1.rop == ReduceOp::Sum && s1.pre.ins.size() == 4 && s1.post.ins.size() == 1 && s1.pre.result == 3 &&
+                   s1.pre.ins[2].op == Op::Sub && s1.pre.ins[3].op == Op::Exp && s1.pre.ins[3].a == 2;
+    if (sum_exp) {
+      const Instr& x = s1.pre.ins[s1.pre.ins[2].a];
+      const Instr& m = s1.pre.ins[s1.pre.ins[2].b];
+      sum_exp = is_load(x, 0) && is_load(m, int(K));
+    }
+    spec.online_max_sum = max_of_x && sum_exp;
+  }
   spec.final = final;
   spec.store_scalars = scalars;
   spec.out_dtype = scalars ? DType::F32 : final.result_dtype();
@@ -766,7 +781,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
     << rb.stages.size() << " operands=" << K + NOUT;
   if (scalars) d << " reductions=" << S;
   if (ragged) d << " ragged";
-  if (streamed) d << " streamed";
+  if (streamed) d << (spec.online_max_sum ? " streamed (max and sum in one pass)" : " streamed");
   r.detail = d.str();
   record(std::move(r), k, row_pack_args(spec, args));
   return true;
