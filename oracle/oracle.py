@@ -28,7 +28,10 @@ entry citing file:line), closed forms (sum of ones, A @ I, norm preservation of
 rope pairs ...), and brute-force index maps for the layout ops.  Functions with
 no reference vector at all: `rope` (the reference has no test for it) and
 `softmax_last_dim` (not in the reference); they are pinned by the mathematics
-only and say so in their docstrings.
+only (parity unpinned at the last bit) and say so in their docstrings.
+`layer_norm` names its broadcast dimensions (RMSNorm as meant); the reference's
+text misplaces the weight on square inputs, which `layer_norm_as_written`
+restates and the tests pin.
 """
 from __future__ import annotations
 
@@ -265,6 +268,19 @@ class OTensor:
         x_normed = f32_self / OTensor(np.broadcast_to(rms.a[:, None], self.a.shape), F32)
         w = OTensor(np.broadcast_to(weight.a[None, :], self.a.shape), weight.a.dtype)
         return x_normed.cast(self.a.dtype) * w
+
+    def layer_norm_as_written(self, weight, eps):
+        """`layer_norm` exactly as the reference's text reads (src/composite/rms_norm.rs:8-15): both broadcasts go
+        through `Tensor::broadcast`, which inserts the new dimension at the FIRST position where the shapes differ
+        (src/map_layout.rs:69-77).  For rows != hidden that is RMSNorm; for a square input (rows == hidden) the
+        weight's shape [hidden] matches the output's first dimension, the new dimension lands at position 1, and the
+        weight ends up indexed by ROW.  `layer_norm` above names its dimensions and is what the HIP path computes;
+        this form exists to pin the difference (tests/test_oracle_kats.py)."""
+        hidden = self.a.shape[-1]
+        f32_self = self.cast(F32)
+        norm_x = (f32_self.sqr().sum(1)) / float(hidden)
+        x_normed = f32_self / (norm_x + eps).sqrt().broadcast(self.a.shape)
+        return x_normed.cast(self.a.dtype) * weight.broadcast(self.a.shape)
 
     def rope(self, cos, sin):
         """y = x*cos + rotate_half(x)*sin, rotate_half(x) = cat(-x2, x1) on the last dim

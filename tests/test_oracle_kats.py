@@ -225,3 +225,21 @@ def test_seeded_generator_is_deterministic_and_well_distributed():
     # SplitMix64 first outputs for seed 0 (published test vector of the algorithm)
     g = SplitMix64(0)
     assert [int(v) for v in g.raw(3)] == [0xE220A8397B1DCDAF, 0x6E789E6AA1B965F4, 0x06C45D188009454F]
+
+
+def test_layer_norm_as_the_reference_writes_it_differs_only_on_square_inputs():
+    # src/composite/rms_norm.rs:13-14 broadcasts through Tensor::broadcast (first differing dimension,
+    # src/map_layout.rs:69-77): RMSNorm for rows != hidden, the weight indexed by ROW for rows == hidden
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((6, 10)).astype(np.float32)
+    w = rng.uniform(0.5, 1.5, 10).astype(np.float32)
+    a = OTensor(x).layer_norm(OTensor(w), 1e-5).to_numpy()
+    b = OTensor(x).layer_norm_as_written(OTensor(w), 1e-5).to_numpy()
+    assert np.array_equal(a, b)
+    sq = rng.standard_normal((10, 10)).astype(np.float32)
+    meant = OTensor(sq).layer_norm(OTensor(w), 1e-5).to_numpy()
+    written = OTensor(sq).layer_norm_as_written(OTensor(w), 1e-5).to_numpy()
+    assert not np.array_equal(meant, written)
+    rms = np.sqrt((sq.astype(np.float64) ** 2).mean(1) + 1e-5)
+    assert np.allclose(meant, sq / rms[:, None] * w[None, :], rtol=1e-6)
+    assert np.allclose(written, sq / rms[:, None] * w[:, None], rtol=1e-6)   # the weight runs down the rows
