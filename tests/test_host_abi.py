@@ -598,6 +598,7 @@ def test_gemm_kernels_use_no_scratch_memory(tmp_path):
         "for dt in (np.float16, np.float32):\n"
         "    for bt in (False, True):\n"
         "        mm(4096, 4096, 128, dt, bt)    # full 256 x 256 tiles\n"
+        "        mm(4096, 4352, 128, dt, bt)    # 272 tiles: the last round in half tiles (f16)\n"
         "        mm(4000, 4104, 136, dt, bt)    # 256 x 256 tiles with ragged edges\n"
         "        mm(512, 512, 256, dt, bt)      # few tiles\n"
         "        mm(300, 264, 2048, dt, bt)     # few ragged tiles, K in slices\n"

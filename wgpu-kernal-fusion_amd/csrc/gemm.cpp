@@ -29,6 +29,9 @@ const char* const kGemmSkinnyTr =
 const char* const kGemmF16T128 =
 #include "kernels/gemm_f16_t128.hip.inc"
     ;
+const char* const kGemmF16Tail =
+#include "kernels/gemm_f16_tail.hip.inc"
+    ;
 // most rows of A the lane-per-column bandwidth kernel takes (accumulators: rows x 8 per lane for f16, rows x 4 for f32;
 // f32 has no MFMA decode kernel for a row-major B, and a 256-row MFMA tile for 32 rows of f32 is 3 times slower still)
 constexpr size_t kSkinnyRowsF16 = 16, kSkinnyRowsF32 = 32;
@@ -353,11 +356,24 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     }
   }
   const bool split = slices > 1;
+  // Full f16 tiles that do not fill a whole number of rounds on the chip (the [2048 x 4096] x [4096 x 11008] MLP
+  // product: 344 tiles on 256 compute units): the tiles of the last, partly filled round are computed as two halves
+  // of 128 rows each by twice as many workgroups, so that round fills twice as many compute units and takes about
+  // half as long (kernels/gemm_f16_tail.hip.inc).
+  size_t ntail = 0, nmain = 0;
+  if (kind == GemmKind::MfmaF16 && !bt && !t128 && !split && batch == 1 && st_.fusion == FusionMode::Tree && st_.gemm_tail) {
+    nmain = tiles / cus * cus;
+    ntail = tiles - nmain;
+    if (nmain == 0 || ntail * 2 > cus) ntail = 0;
+  }
+  const bool tail = ntail > 0;
   TensorData out = split ? alloc(slices_shape(slices), DType::F32, false) : alloc(out_shape, a.dtype, false);
   std::string sig = t128 ? std::string("gemm|gfx950|f16|mfma32x32x16|128x128x64|w2x2|edge") : gemm_signature(kind, a.dtype);
   if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
   if (bt) sig += "|bt";
+  if (tail) sig += "|last round in half tiles";
   wkf_kernel* k = kernel(sig, [&] {
+    if (tail) return std::string(kGemmF16Tail);
     std::string src = bt ? "#define WKF_BT 1\n" : "";
     if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + kGemmF16T128;
     if (!split) return src + gemm_source(kind, a.dtype);
@@ -374,6 +390,12 @@ TensorData Resolver::run_matmul(const NodeP& n) {
             uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(kchunk)};
   std::vector<unsigned char> bytes(sizeof(args));
   memcpy(bytes.data(), &args, sizeof(args));
+  if (tail) {
+    const uint32_t extra[2] = {uint32_t(nmain), uint32_t(ntail)};
+    const size_t at = bytes.size();
+    bytes.resize(at + sizeof(extra));
+    memcpy(bytes.data() + at, extra, sizeof(extra));
+  }
 
   LaunchRecord r;
   r.kind = "gemm";
@@ -385,7 +407,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     if (r.grid[1] > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many rows for the generic kernel");
   } else {
     if (tiles > 0x7fffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
-    r.grid[0] = uint32_t(tiles);
+    r.grid[0] = uint32_t(tail ? nmain + 2 * ntail : tiles);
     r.grid[1] = uint32_t(slices);
   }
   r.grid[2] = uint32_t(batch);
@@ -394,6 +416,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (!t128 && (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge)) d << " edge";
   if (bt) d << " B^T";
   if (split) d << " slices=" << slices;
+  if (tail) d << ", last round: " << ntail << " tiles as " << 2 * ntail << " halves of 128 rows";
   if (batch > 1) d << " batch=" << batch;
   r.detail = d.str();
   record(std::move(r), k, bytes);
