@@ -126,6 +126,21 @@ def measure_batch(w, dev, wl, steps, warmup):
         lib.wkf_timer_destroy(timer)
 
 
+def settle(dev, wl, seconds=0.3):
+    """Runs the workload untimed for `seconds`: after uploads and an idle spell the GPU takes tens of milliseconds to
+    reach its working clocks.  Not part of any measurement (the W warm-up steps of each measurement still run)."""
+    dev.set_timing(False)
+    t_end = time.perf_counter() + seconds
+    i = 0
+    while time.perf_counter() < t_end:
+        wl.step(i)
+        i += 1
+        if i % 50 == 0:
+            dev.sync()
+    dev.sync()
+    dev.set_timing(True)
+
+
 def measure_wall(dev, wl, steps, warmup):
     """Wall-clock seconds for `steps` steps, no per-launch events, synchronised on both sides."""
     dev.set_timing(False)
@@ -348,6 +363,7 @@ def copy_ceiling(w, dev):
     x = w.Tensor.new(dev, np.zeros((1 << 28,), dtype=np.float32))
     t = x.resize([1 << 28])  # resize to the same shape = one dense copy kernel
     wl = Workload("copy", [[t]], 2 * (1 << 30), "GB/s", HBM_PEAK_GBS)
+    settle(dev, wl)
     k, med, _ = measure_kernels(dev, wl, 10, 3)
     return round(wl.work / med * 1e-3, 1)
 
@@ -410,18 +426,11 @@ def profile_one(w, dev, seeded, key, launches, warm_ms):
         if key not in wls:
             sys.exit(f"bench.py --profile: unknown workload {key!r}; group {group!r} has: " + ", ".join(wls))
         wl = wls[key]
-    dev.set_timing(False)
-    t_end = time.perf_counter() + warm_ms * 1e-3
-    i = 0
-    while time.perf_counter() < t_end:
-        wl.step(i)
-        i += 1
-        if i % 50 == 0:
-            dev.sync()
-    dev.sync()
+    if warm_ms > 0:
+        settle(dev, wl, warm_ms * 1e-3)
     us = measure_batch(w, dev, wl, launches, 10)
     scale = 1e-3 if wl.unit == "GB/s" else 1e-6
-    print(json.dumps({"profile": key, "warm_steps": i + 10, "name": wl.name, "launches": launches, "us_per_step": round(us, 2),
+    print(json.dumps({"profile": key, "name": wl.name, "launches": launches, "us_per_step": round(us, 2),
                       "achieved": round(wl.work / us * scale, 1), "unit": wl.unit, "frac": round(wl.work / us * scale / wl.peak, 4),
                       "work_per_step": wl.work}))
 
@@ -639,6 +648,7 @@ def main():
     with_cpu = not args.no_cpu
     head = build_workloads(w, dev, seeded, {"c2"}, with_cpu)
     wl = head["c2"]
+    settle(dev, wl)
     kernels, _, _ = measure_kernels(dev, wl, args.steps, args.warmup)
     wall = measure_wall(dev, wl, args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
@@ -685,6 +695,7 @@ def main():
             for key, one in wls.items():
                 if key == "c2":
                     continue
+                settle(dev, one)  # the CPU port and the uploads before this row left the GPU idle
                 measured = measure_kernels(dev, one, steps, warm)
                 wall_s = measure_wall(dev, one, steps, 5)
                 batch_us = round(measure_batch(w, dev, one, steps, 5), 2)
