@@ -313,6 +313,24 @@ def test_reductions_of_views_and_rank0(gpu):
     assert got[5].shape == () and got[6].shape == ()
 
 
+def test_reductions_of_views_with_many_outer_dimensions(gpu):
+    # a 5-D slice leaves four outer dimensions that do not merge: more than the reduce kernels decode, so the view is
+    # copied into a dense buffer first (the reference's reduce takes any rank, src/reduce.rs:83-281)
+    a = data((6, 6, 6, 6, 6), -1, 1, np.float32, 16)
+    api = HipAPI(gpu)
+    cut = [(1, 5)] * 5
+
+    def progs(t):
+        v = t.slice(cut)
+        return [v.sum(4), v.max(0), (v * 2.0).exp().sum(2), v.transpose(0, 4).sum(1)]
+
+    got = hip_values_many(progs(api.tensor(a)))
+    want = progs(OTensor(a))
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert g.shape == w.to_numpy().shape
+        assert np.allclose(g, w.to_numpy(), rtol=1e-5, atol=1e-6), f"5-D view reduce {i}"
+
+
 def test_long_axis_reductions_of_views(gpu):
     api = HipAPI(gpu)
     a = data((4096, 96), -1, 1, np.float32, 16)
