@@ -561,8 +561,8 @@ def test_row_kernels_on_rows_that_do_not_split_evenly(gpu, rows, n, dtype):
     assert np.allclose(got[2].astype(np.float64), total, rtol=1e-5 if dtype == np.float32 else 4e-3)
 
 
-LONG_ROWS = [(128, 100003, np.float32), (130, 262144, np.float32), (129, 70000, np.float32), (128, 140002, np.float16),
-             (131, 131080, np.float16)]
+LONG_ROWS = [(256, 100003, np.float32), (258, 131076, np.float32), (257, 70000, np.float32), (256, 140002, np.float16),
+             (261, 131080, np.float16)]
 
 
 @pytest.mark.parametrize("rows,n,dtype", LONG_ROWS, ids=[f"{r}x{n}_{np.dtype(d).name}" for r, n, d in LONG_ROWS])
@@ -598,15 +598,72 @@ def test_rows_longer_than_a_blocks_registers_stay_one_kernel(gpu, rows, n, dtype
         assert np.allclose(se, ref, rtol=1e-5)
 
 
-def test_few_long_rows_fold_across_the_grid(gpu):
-    # with only a few rows a block per row would leave most compute units idle: those keep the reductions that are
-    # folded across the whole grid (several launches), with the same values
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+@pytest.mark.parametrize("rows,n", [(5, 100003), (64, 65540), (1, 1 << 20), (100, 70000), (127, 65600), (3, 70001)])
+def test_few_long_rows_are_split_into_parts(gpu, rows, n, dtype):
+    # with only a few rows a block per row would leave most compute units idle: every row is cut into parts with a
+    # block each and every stage becomes one launch that leaves its parts' values to the next (softmax: the online
+    # pair of max and sum, then the result = two launches; layer_norm: three).  The reference's reduce takes any
+    # length in one kernel (src/reduce.rs:340-350).
+    if dtype == np.float16:
+        # as many bytes as the f32 case, so that the rows are too long for a block's registers, but no more
+        # than about 390 000 elements: beyond that sum(exp(x - max)) of these inputs overflows f16
+        n = min(2 * n, 1 << 18)
+    x = data((rows, n), -3, 3, dtype, rows * 13 + n)
+    w = data((n,), 0.5, 1.5, dtype, n + 2)
+    api = HipAPI(gpu)
+    tx, tw = api.tensor(x), api.tensor(w)
+    ox, ow = OTensor(x), OTensor(w)
+    progs = [tx.softmax_last_dim()]
+    want = [ox.softmax_last_dim().to_numpy()]
+    launches = [2]
+    if dtype == np.float32:
+        progs.append(tx.layer_norm(tw, 1e-5))
+        want.append(ox.layer_norm(ow, 1e-5).to_numpy())
+        launches.append(2)
+    got = hip_values_many(progs)
+    for p, count in zip(progs, launches):
+        ks = p.kernels()
+        assert [k.kind for k in ks] == ["row"] * count, [(k.kind, k.detail) for k in ks]
+        assert all("rows split in" in k.detail for k in ks), [k.detail for k in ks]
+    rtol = 1e-5 if dtype == np.float32 else 2e-3
+    for i in range(len(got)):
+        assert got[i].shape == want[i].shape
+        assert np.allclose(got[i].astype(np.float64), want[i].astype(np.float64), rtol=rtol, atol=1e-9 if dtype == np.float32 else 1e-7), i
+    assert np.allclose(got[0].astype(np.float64).sum(1), 1.0, atol=1e-5 if dtype == np.float32 else 5e-2)
+    assert np.array_equal(np.argmax(got[0], 1), np.argmax(x, 1))
+
+
+def test_split_rows_of_a_view_and_with_stages_that_do_not_pair(gpu):
+    # the operand is a column block of a wider matrix (row stride != row length)
+    big = data((6, 3 * 100000), -2, 2, np.float32, 5)
+    api = HipAPI(gpu)
+    w = data((100000,), 0.5, 1.5, np.float32, 6)
+    t = api.tensor(big).slice([(0, 6), (100000, 200000)]).layer_norm(api.tensor(w), 1e-5)
+    got = hip_values(t)
+    want = OTensor(big).slice([(0, 6), (100000, 200000)]).layer_norm(OTensor(w), 1e-5).to_numpy()
+    assert len(t.kernels()) == 2 and all("rows split in" in k.detail for k in t.kernels()), [k.detail for k in t.kernels()]
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-7)
+    # softmax of 2x: the maximum is not of the operand itself, so max and sum stay passes of their own (three launches)
+    x = data((9, 90000), -3, 3, np.float32, 8)
+    t = (api.tensor(x) * 0.5).softmax_last_dim()
+    got = hip_values(t)
+    want = (OTensor(x) * 0.5).softmax_last_dim().to_numpy()
+    ks = t.kernels()
+    assert len(ks) == 3 and all("rows split in" in k.detail and "in one pass" not in k.detail for k in ks), [k.detail for k in ks]
+    assert np.allclose(got, want, rtol=1e-5, atol=1e-9)
+
+
+def test_few_long_rows_of_stored_reductions_fold_across_the_grid(gpu):
+    # reductions that are stored (no result rows) of a few long rows keep the kernels that fold across the whole grid
     x = data((5, 100003), -3, 3, np.float32, 77)
     api = HipAPI(gpu)
-    t = api.tensor(x).softmax_last_dim()
-    got = hip_values(t)
-    assert len(t.kernels()) > 1
-    assert np.allclose(got, OTensor(x).softmax_last_dim().to_numpy(), rtol=1e-5, atol=1e-9)
+    t = api.tensor(x)
+    pair = [t.max(1), (t.clone() - 1.0).exp().sum(1)]
+    m, se = hip_values_many(pair)
+    assert np.array_equal(m, x.max(1))
+    ref = np.exp((x - np.float32(1.0)).astype(np.float64)).astype(np.float32).astype(np.float64).sum(1)
+    assert np.allclose(se, ref, rtol=1e-5)
 
 
 # ---- the benchmark configurations at full size ------------------------------------------------------------------------------

@@ -399,9 +399,19 @@ def test_row_kernel_takes_rows_that_do_not_split_evenly(wkf, planner):
     assert "vec=8" in detail((8, 2880), np.float16, sm) and "vec=4" in detail((8, 11004), np.float16, sm)
     # rows of a view that start off the vector grid take narrower vectors instead of three kernels
     assert "vec=1" in detail((8, 4096), np.float32, lambda t: t.slice([(0, 8), (1, 4095)]).softmax_last_dim())
-    # beyond what 1024 lanes hold in registers the reductions and the map run on their own
+    # beyond what 1024 lanes hold in registers a few rows are split into parts: one launch for the online pair of
+    # max and sum over every part, one that folds a row's parts and writes the result
     long_rows = _x(wkf, planner, (2, 65537), np.float32).softmax_last_dim()
-    assert _kinds(long_rows) == ["red_row", "red_row", "map"]
+    assert _kinds(long_rows) == ["row", "row"]
+    details = [k.detail for k in long_rows.kernels()]
+    assert details[0].endswith("streamed (max and sum in one pass), rows split in 65 parts of 1024 vectors: launch 1 of 2"), details
+    assert details[1].endswith("launch 2 of 2") and long_rows.kernels()[0].signature.endswith("|split0")
+    assert long_rows.kernels()[1].signature.endswith("|split2")
+    # 256 rows or more stream with a block per row, in one launch
+    many = _x(wkf, planner, (256, 65537), np.float32).softmax_last_dim()
+    assert _kinds(many) == ["row"] and many.kernels()[0].detail.endswith("streamed (max and sum in one pass)")
+    # rows that are short but too many vectors for the lanes' registers (fewer than 1024 vectors never are) stay decomposed
+    assert _kinds(_x(wkf, planner, (2, 70000), np.float32).max(1)) == ["red_row", "red_row"]
 
 
 def test_f16_column_max_with_a_post_op_compiles(wkf, planner):

@@ -846,6 +846,7 @@ std::string row_signature(const RowSpec& s) {
   if (s.ragged) o << "|ragged";
   if (s.streamed) o << "|streamed";
   if (s.online_max_sum) o << "|online";
+  if (s.split) o << "|split" << s.split_phase;
   return o.str();
 }
 
@@ -880,7 +881,8 @@ std::string row_source(const RowSpec& s) {
     if (round_h) o << kRoundH;
   }
   o << kRowHelpers;
-  o << "struct Args { void* p[" << K + NOUT << "]; u32 nrows; " << (s.ragged || s.streamed ? "u32 nvec; " : "") << "u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
+  o << "struct Args { void* p[" << K + NOUT + (s.split ? 1 : 0) << "]; u32 nrows; " << (s.ragged || s.streamed ? "u32 nvec; " : "") << (s.split ? "u32 parts; u32 chunk; " : "")
+    << "u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
     << "]; u32 ostride[" << K + NOUT << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
   // operand types as every program sees them: the K full operands, then one scalar per earlier stage
   std::vector<DType> types;
@@ -896,7 +898,8 @@ std::string row_source(const RowSpec& s) {
   o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") WKF_ENTRY(const Args a) {\n";
   if (T > 64) o << "  __shared__ float wkf_partial[" << std::max(1, S) << "][" << B / 64 << "];\n";
   o << "  const u32 t = threadIdx.x % " << T << "u;\n";
-  o << "  const u32 row_raw = blockIdx.x * " << RPB << "u + threadIdx.x / " << T << "u;\n";
+  if (s.split) o << "  const u32 part = blockIdx.x % a.parts;\n  const u32 row_raw = blockIdx.x / a.parts;\n";
+  else o << "  const u32 row_raw = blockIdx.x * " << RPB << "u + threadIdx.x / " << T << "u;\n";
   o << "  const bool live = row_raw < a.nrows;\n";
   o << "  const u32 row = live ? row_raw : 0u;\n";
   if (s.ragged) o << "  const bool last_ok = t + " << (NV - 1) * T << "u < a.nvec;  // this lane's last vector lies inside the row\n";
@@ -932,9 +935,13 @@ std::string row_source(const RowSpec& s) {
       for (int q = 0; q < nscalars; q++) c << "r" << q << ", ";
       return c.str();
     };
+    // A split kernel walks its part of the row, [part * chunk, (part + 1) * chunk); an unsplit one all of it.
+    if (s.split) o << "  const u32 lo = part * a.chunk;\n  const u32 hi = min(a.nvec, lo + a.chunk);\n";
+    else o << "  const u32 lo = 0u;\n  const u32 hi = a.nvec;\n";
+    const std::string loop = "  for (u32 base = lo; base < hi; base += " + std::to_string(T * U) + "u) {\n";
     // `last`: the final pass streams (nothing reads the row again); earlier passes leave it in the caches
     auto emit_loads = [&](bool last) {
-      for (int u = 0; u < U; u++) o << "    const u32 j" << u << " = base + t + " << u * T << "u; const bool ok" << u << " = j" << u << " < a.nvec;\n";
+      for (int u = 0; u < U; u++) o << "    const u32 j" << u << " = base + t + " << u * T << "u; const bool ok" << u << " = j" << u << " < hi;\n";
       for (int k = 0; k < K; k++) {
         if (s.in[k].axis_stride == 0) continue;
         std::string vt = vtype(s.in[k].dtype, V);
@@ -948,25 +955,62 @@ std::string row_source(const RowSpec& s) {
     const bool last_is_stage = s.store_scalars;
     auto block_fold = [&](int k) {  // acc<k> of every lane -> the row's value in every lane
       o << "  acc" << k << " = wkf_lanes_fold_with<64>(acc" << k << ", fold" << k << ");\n";
-      o << "  if ((threadIdx.x & 63u) == 0u) wkf_partial[" << k << "][threadIdx.x >> 6] = acc" << k << ";\n";
-      o << "  __syncthreads();\n";
-      o << "  acc" << k << " = wkf_partial[" << k << "][0];\n";
-      o << "  for (u32 w = 1; w < " << T / 64 << "u; w++) acc" << k << " = fold" << k << "(wkf_partial[" << k << "][w], acc" << k << ");\n";
+      if (T > 64) {
+        o << "  if ((threadIdx.x & 63u) == 0u) wkf_partial[" << k << "][threadIdx.x >> 6] = acc" << k << ";\n";
+        o << "  __syncthreads();\n";
+        o << "  acc" << k << " = wkf_partial[" << k << "][0];\n";
+        o << "  for (u32 w = 1; w < " << T / 64 << "u; w++) acc" << k << " = fold" << k << "(wkf_partial[" << k << "][w], acc" << k << ");\n";
+      }
     };
-    if (s.online_max_sum) {
+    auto emit_post = [&](int k) {
+      o << "  const " << ctype(s.stages[k].post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(s.stages[k].pre.result_dtype())
+        << ")acc" << k << ", a.c + " << post_off[k] << ");\n";
+    };
+    for (int k = 0; k < S; k++) {
+      const bool online = s.online_max_sum && k < 2;
+      o << "  float acc" << k << " = " << seed_text(online ? (k == 0 ? ReduceOp::Max : ReduceOp::Sum) : s.stages[k].rop) << ";\n";
+      o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(online ? (k == 0 ? ReduceOp::Max : ReduceOp::Sum) : s.stages[k].rop)
+        << "; };\n";
+    }
+    // Split rows: stage k of part q of a row leaves its folded value in wp[(k * nrows + row) * parts + q]; the
+    // kernels after it fold a row's `parts` values (one per lane) before they start.  The sums of an online pair
+    // are relative to their own part's maximum and are rescaled to the row's when they are combined.
+    const int first = s.split ? s.split_phase : 0;  // the first stage this kernel folds itself
+    if (s.split) {
+      o << "  float* const wp = (float*)a.p[" << K + NOUT << "];\n";
+      auto part_at = [&](int k) { return "wp[(" + std::to_string(k) + "u * a.nrows + row) * a.parts + t]"; };
+      for (int k = 0; k < first; k++) {
+        if (s.online_max_sum && k == 0) {
+          o << "  const float part_max = t < a.parts ? " << part_at(0) << " : acc0;\n  acc0 = part_max;\n";
+          block_fold(0);
+          o << "  if (t < a.parts) acc1 = " << part_at(1) << " * expf(part_max - acc0);\n";
+          block_fold(1);
+          emit_post(0);
+          emit_post(1);
+          k = 1;
+          continue;
+        }
+        o << "  if (t < a.parts) acc" << k << " = " << part_at(k) << ";\n";
+        block_fold(k);
+        emit_post(k);
+      }
+    }
+    auto leave_parts = [&](int k0, int k1) {  // a split kernel ends here: lane 0 stores what this part folded
+      o << "  if (t == 0u) {\n";
+      for (int k = k0; k <= k1; k++) o << "    wp[(" << k << "u * a.nrows + row) * a.parts + part] = acc" << k << ";\n";
+      o << "  }\n}\n";
+    };
+    if (s.online_max_sum && first == 0) {
       // stages 0 and 1 in one pass: every lane keeps a running maximum m and the sum of exp(x - m) over what it
       // has seen; when m grows the sum is rescaled by exp(old m - new m).  Lanes are combined the same way.
       const char* mt = ctype(s.stages[0].post.result_dtype());
-      o << "  float acc0 = " << seed_text(ReduceOp::Max) << ", acc1 = 0.0f;\n";
-      o << "  auto fold0 = [](float v, float a) { return fmaxf(v, a); };\n";
-      o << "  auto fold1 = [](float v, float a) { return v + a; };\n";
-      o << "  for (u32 base = 0; base < a.nvec; base += " << T * U << "u) {\n";
+      o << loop;
       emit_loads(last_is_stage && S == 2);
       for (int u = 0; u < U; u++) {
         o << "    if (ok" << u << ") {\n";
         o << "      float cm = acc0;\n";
         for (int e = 0; e < V; e++) o << "      cm = fmaxf((float)wkf_pre0(" << sargs(u, e, 0) << "a.c + " << pre_off[0] << "), cm);\n";
-        o << "      acc1 *= expf(acc0 - cm);\n      acc0 = cm;\n";
+        o << "      if (cm > acc0) {  // rare after the first steps of a row: exp(0) = 1 would change nothing\n        acc1 *= expf(acc0 - cm);\n        acc0 = cm;\n      }\n";
         o << "      const " << mt << " r0 = wkf_post0((" << ctype(s.stages[0].pre.result_dtype()) << ")cm, a.c + " << post_off[0] << ");\n";
         for (int e = 0; e < V; e++) o << "      acc1 += (float)wkf_pre1(" << sargs(u, e, 1) << "a.c + " << pre_off[1] << ");\n";
         o << "    }\n";
@@ -976,15 +1020,15 @@ std::string row_source(const RowSpec& s) {
       block_fold(0);
       o << "  acc1 *= expf(lane_max - acc0);\n";
       block_fold(1);
-      for (int k = 0; k < 2; k++)
-        o << "  const " << ctype(s.stages[k].post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(s.stages[k].pre.result_dtype())
-          << ")acc" << k << ", a.c + " << post_off[k] << ");\n";
+      if (s.split) {
+        leave_parts(0, 1);
+        return o.str();
+      }
+      emit_post(0);
+      emit_post(1);
     }
-    for (int k = s.online_max_sum ? 2 : 0; k < S; k++) {
-      const RowStage& st = s.stages[k];
-      o << "  float acc" << k << " = " << seed_text(st.rop) << ";\n";
-      o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(st.rop) << "; };\n";
-      o << "  for (u32 base = 0; base < a.nvec; base += " << T * U << "u) {\n";
+    for (int k = std::max(first, s.online_max_sum ? 2 : 0); k < S; k++) {
+      o << loop;
       emit_loads(last_is_stage && k == S - 1);
       for (int u = 0; u < U; u++) {
         o << "    if (ok" << u << ") {\n";
@@ -994,8 +1038,11 @@ std::string row_source(const RowSpec& s) {
       }
       o << "  }\n";
       block_fold(k);
-      o << "  const " << ctype(st.post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(st.pre.result_dtype()) << ")acc" << k
-        << ", a.c + " << post_off[k] << ");\n";
+      if (s.split) {
+        leave_parts(k, k);
+        return o.str();
+      }
+      emit_post(k);
     }
     if (s.store_scalars) {
       o << "  if (live && t == 0u) {\n";
@@ -1009,7 +1056,7 @@ std::string row_source(const RowSpec& s) {
     const char* sot = ctype(s.out_dtype);
     std::string ovt = vtype(s.out_dtype, V);
     o << "  " << sot << "* qo = ((" << sot << "*)a.p[" << K << "]) + (" << base_expr(K) << ");\n";
-    o << "  for (u32 base = 0; base < a.nvec; base += " << T * U << "u) {\n";
+    o << loop;
     emit_loads(true);
     for (int u = 0; u < U; u++) {
       o << "    if (live && ok" << u << ") {\n      " << ovt << " ov;\n";
@@ -1106,12 +1153,16 @@ std::string row_source(const RowSpec& s) {
 std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a) {
   const size_t K = s.in.size(), Ro = size_t(s.outer_rank);
   const size_t NP = K + (s.store_scalars ? s.stages.size() : 1);
-  if (a.ptrs.size() != NP || a.oshape.size() != Ro || a.offsets.size() != NP || a.ostrides.size() != NP)
+  if (a.ptrs.size() != NP + (s.split ? 1 : 0) || a.oshape.size() != Ro || a.offsets.size() != NP || a.ostrides.size() != NP)
     throw Error(WKF_ERR_INVALID_ARG, "row_pack_args: argument arity does not match the kernel");
   std::vector<unsigned char> b;
   for (void* p : a.ptrs) putp(b, p);
   put32(b, a.nrows);
   if (s.ragged || s.streamed) put32(b, a.nvec);
+  if (s.split) {
+    put32(b, a.parts);
+    put32(b, a.chunk);
+  }
   for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? a.oshape[d] : 1);
   for (uint32_t v : a.offsets) put32(b, v);
   for (const auto& st : a.ostrides) {

@@ -149,6 +149,13 @@ struct RowSpec {
   // with a running maximum (the running sum is rescaled by exp(old max - new max) whenever the maximum grows), so
   // the row is read twice in all instead of three times
   bool online_max_sum = false;
+  // split (streamed rows only, with a `final`): too few rows to occupy the chip with a block each.  Every row is cut
+  // into `parts` parts (a launch argument) of `chunk` vectors, one block of T lanes per part, and the stages become
+  // kernels of their own: kernel `split_phase` = k < stages folds stage k over its part and leaves the value in a
+  // buffer of [stages][rows][parts] floats (the extra, last pointer argument); kernel `split_phase` = stages writes
+  // the result.  Each first folds the parts of the stages before it.  An online pair is one kernel (phase 0).
+  bool split = false;
+  int split_phase = 0;
   std::vector<ReduceOperandSpec> in;    // axis_stride 1 (row in registers) or 0 (one scalar per row)
   std::vector<RowStage> stages;
   Program final;                        // same operand numbering as a stage's pre
@@ -161,9 +168,10 @@ struct RowSpec {
 std::string row_signature(const RowSpec& s);
 std::string row_source(const RowSpec& s);
 struct RowArgs {
-  std::vector<void*> ptrs;                        // inputs..., out (store_scalars: one out per stage)
+  std::vector<void*> ptrs;                        // inputs..., out (store_scalars: one out per stage)[, the parts of a split row]
   uint32_t nrows;
-  uint32_t nvec = 0;                              // ragged kernels only: vectors per row
+  uint32_t nvec = 0;                              // ragged and streamed kernels only: vectors per row
+  uint32_t parts = 0, chunk = 0;                  // split kernels only: parts per row, vectors per part
   std::vector<uint32_t> oshape;
   std::vector<uint32_t> offsets;                  // per operand incl. outputs
   std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. outputs, per outer dim

@@ -697,17 +697,31 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   size_t nrows = 1;
   for (size_t d : out_shape) nrows *= d;
   if (nrows > 0xffffffffull) return false;
-  bool streamed = false;
+  bool streamed = false, split = false;
+  size_t parts = 1, chunk = 0;
   if (NV > max_nv || NV * V * K > 128) {
     // The row does not fit the registers of a block.  With enough rows to occupy the chip, one block per row
     // streams its row once per stage and once more for the result, in ONE launch; the passes after the first
     // find the row in the caches when it fits them.  With only a few rows a block per row would leave most
-    // compute units idle: the caller then folds each reduction across the whole grid instead (several launches).
-    if (nrows < st_.row_stream_min_rows || nvec < 1024) return false;
+    // compute units idle: every row is then cut into parts with a block each and every stage becomes a launch
+    // of its own, which leaves its parts' values to the next (softmax: two launches).  Reductions that are
+    // stored (no result rows) are folded across the whole grid by the caller instead.
+    if (nvec < 1024) return false;
     streamed = true;
     ragged = false;
-    T = 1024;
     NV = std::max<size_t>(1, std::min<size_t>(4, 8 / std::max<size_t>(1, K)));  // vectors in flight per lane and operand
+    if (nrows >= st_.row_stream_min_rows) {
+      T = 1024;
+    } else {
+      if (scalars || !st_.row_split) return false;
+      split = true;
+      T = 256;
+      // about eight blocks per compute unit, every part a whole number of steps of the block, at most one part per lane
+      const size_t step = size_t(T) * NV;
+      const size_t want = std::min<size_t>(size_t(T), std::max<size_t>(1, 2048 / nrows));
+      chunk = ((nvec + want - 1) / want + step - 1) / step * step;
+      parts = (nvec + chunk - 1) / chunk;
+    }
   }
 
   // operand numbering: full operands 0..K-1, then the scalars
@@ -768,22 +782,48 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   }
   args.consts.insert(args.consts.end(), final.consts.begin(), final.consts.end());
 
-  std::string sig = row_signature(spec);
-  wkf_kernel* k = kernel(sig, [&] { return row_source(spec); });
-  LaunchRecord r;
-  r.kind = "row";
-  r.signature = sig;
-  const size_t rpb = size_t(spec.block / T);
-  r.grid[0] = to_u32((nrows + rpb - 1) / rpb, "grid");
-  r.block[0] = uint32_t(spec.block);
   std::ostringstream d;
   d << "rows=" << nrows << " n=" << n << " vec=" << V << " threads_per_row=" << T << " vectors_per_lane=" << NV << " stages="
     << rb.stages.size() << " operands=" << K + NOUT;
   if (scalars) d << " reductions=" << S;
   if (ragged) d << " ragged";
   if (streamed) d << (spec.online_max_sum ? " streamed (max and sum in one pass)" : " streamed");
-  r.detail = d.str();
-  record(std::move(r), k, row_pack_args(spec, args));
+  const size_t rpb = size_t(spec.block / T);
+  if (!split) {
+    std::string sig = row_signature(spec);
+    wkf_kernel* k = kernel(sig, [&] { return row_source(spec); });
+    LaunchRecord r;
+    r.kind = "row";
+    r.signature = sig;
+    r.grid[0] = to_u32((nrows + rpb - 1) / rpb, "grid");
+    r.block[0] = uint32_t(spec.block);
+    r.detail = d.str();
+    record(std::move(r), k, row_pack_args(spec, args));
+    return true;
+  }
+  // split rows: one launch per stage (an online pair counts as one), then the launch that writes the rows
+  TensorData part_values = alloc({S, nrows, parts}, DType::F32, false);
+  args.ptrs.push_back(element_ptr(part_values));
+  args.parts = to_u32(parts, "parts");
+  args.chunk = to_u32(chunk, "chunk");
+  spec.split = true;
+  std::vector<int> phases;
+  for (size_t p = 0; p <= S; p++)
+    if (!(spec.online_max_sum && p == 1)) phases.push_back(int(p));
+  for (size_t i = 0; i < phases.size(); i++) {
+    spec.split_phase = phases[i];
+    std::string sig = row_signature(spec);
+    wkf_kernel* k = kernel(sig, [&] { return row_source(spec); });
+    LaunchRecord r;
+    r.kind = "row";
+    r.signature = sig;
+    r.grid[0] = to_u32(nrows * parts, "grid");
+    r.block[0] = uint32_t(spec.block);
+    std::ostringstream dd;
+    dd << d.str() << ", rows split in " << parts << " parts of " << chunk << " vectors: launch " << i + 1 << " of " << phases.size();
+    r.detail = dd.str();
+    record(std::move(r), k, row_pack_args(spec, args));
+  }
   return true;
 }
 

@@ -41,7 +41,8 @@ struct Settings {
   int skinny_tr_rows = 0;         // fewest rows of A for the MFMA decode kernel on row-major B; 0 = chosen (WKF_SKINNY_TR_ROWS overrides)
   int skinny_blocks = 0;          // workgroups the decode-sized mat_mul kernels aim for; 0 = chosen (WKF_SKINNY_BLOCKS overrides)
   int reduce_unroll = 0;          // loads in flight per lane in row reduces; 0 = chosen (WKF_REDUCE_UNROLL overrides)
-  size_t row_stream_min_rows = 128;  // fewest rows for the one-launch kernel that streams rows longer than a block's registers (WKF_ROW_STREAM_MIN_ROWS)
+  bool row_split = true;             // rows too long for a block's registers and too few to stream with a block each: one launch per stage over parts of rows (WKF_ROW_SPLIT=0: fold each reduction across the grid instead)
+  size_t row_stream_min_rows = 256;  // fewest rows for the one-launch kernel that streams rows longer than a block's registers (WKF_ROW_STREAM_MIN_ROWS)
 };
 
 // The iteration space of one kernel seen by all of its operands at once:

@@ -116,6 +116,7 @@ Settings settings_for(wkf_device* dev) {
     }
     if (const char* u = getenv("WKF_GEMM_T128")) st.gemm_t128 = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_TAIL")) st.gemm_tail = atoi(u) != 0;
+    if (const char* u = getenv("WKF_ROW_SPLIT")) st.row_split = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_STREAM_MIN_ROWS")) st.row_stream_min_rows = size_t(std::max(1ll, atoll(u)));
     if (const char* u = getenv("WKF_SKINNY_TR_ROWS")) {
       int v = atoi(u);
