@@ -80,7 +80,7 @@ class Workload:
 
 
 def measure_kernels(dev, wl, steps, warmup):
-    """Per-kernel GPU time (hipEvent pair around each launch) over `steps` steps after `warmup` untimed ones:
+    """Per-kernel GPU time (a hipEvent pair carried by each dispatch: the kernel's own begin to end) over `steps` steps after `warmup` untimed ones:
     the median and the minimum per kernel, and of the step's total."""
     dev.set_timing(True)
     for i in range(warmup):

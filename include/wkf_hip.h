@@ -105,7 +105,13 @@ int wkf_module_stats(wkf_device* dev, uint64_t* compiled, uint64_t* disk_hits, u
  * dispatch_workgroups, src/kernel.rs:375-384.  `args` is the packed kernel
  * argument block (it also replaces the per-tensor uniform buffers of
  * src/kernel.rs:274-361).  hipModuleLaunchKernel on the device stream; when
- * `timer` is non-NULL a hipEvent pair is recorded around the launch. */
+ * `timer` is non-NULL the launch carries the timer's two events in the dispatch
+ * itself (hipExtModuleLaunchKernel): they take the kernel's own begin and end
+ * timestamps, as the reference's timestamp queries around a compute pass do
+ * (src/query.rs:50-126), and put nothing else on the stream.  With
+ * WKF_TIMER_EVENTS=1 in the environment, or a grid of more than 2^32 - 1
+ * work-items in one dimension, two events are recorded around the launch
+ * instead (about 2.5 us more per launch, and the gap to the kernel before). */
 int wkf_launch(wkf_device* dev, wkf_kernel* kernel, const uint32_t grid[3],
                const uint32_t block[3], uint32_t dyn_lds_bytes, const void* args,
                size_t arg_bytes, wkf_timer* timer);

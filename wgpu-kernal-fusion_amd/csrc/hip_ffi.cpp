@@ -5,6 +5,7 @@
 #include "wkf_hip.h"
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <hip/hiprtc.h>
 
 #include <dlfcn.h>
@@ -121,6 +122,8 @@ struct wkf_device {
   // buffers handed out and not yet released; a destroy with some still alive is deferred to the last release
   size_t live_buffers = 0;
   bool closing = false;
+  // timed launches take their events inside the dispatch (WKF_TIMER_EVENTS=1: two recorded events around it instead)
+  bool timer_in_dispatch = [] { const char* e = getenv("WKF_TIMER_EVENTS"); return !(e && atoi(e) != 0); }();
   // events of destroyed timers, handed out again by wkf_timer_create: a timed launch costs two event
   // records, not two event creations and destructions
   std::vector<hipEvent_t> free_events;
@@ -574,6 +577,17 @@ int wkf_launch(wkf_device* dev, wkf_kernel* kernel, const uint32_t grid[3], cons
   size_t size = arg_bytes;
   void* config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void*>(args), HIP_LAUNCH_PARAM_BUFFER_SIZE, &size,
                     HIP_LAUNCH_PARAM_END};
+  // A timed launch carries its two events in the dispatch itself: they take the kernel's own begin and end
+  // timestamps (what a profiler's kernel trace shows, and what the reference's timestamp queries around a compute
+  // pass measure, src/query.rs:50-126) and put no packets of their own on the stream.  That call takes the grid in
+  // work-items, 32 bits per dimension; a larger grid is bracketed by two recorded events instead.
+  const uint64_t gx = uint64_t(grid[0]) * block[0], gy = uint64_t(grid[1]) * block[1], gz = uint64_t(grid[2]) * block[2];
+  if (timer && dev->timer_in_dispatch && gx <= 0xffffffffull && gy <= 0xffffffffull && gz <= 0xffffffffull) {
+    WKF_HIP_CHECK(hipExtModuleLaunchKernel(kernel->function, uint32_t(gx), uint32_t(gy), uint32_t(gz), block[0], block[1], block[2],
+                                           dyn_lds_bytes, dev->stream, nullptr, config, timer->begin, timer->end, 0));
+    timer->recorded = true;
+    return WKF_OK;
+  }
   if (timer) WKF_HIP_CHECK(hipEventRecord(timer->begin, dev->stream));
   WKF_HIP_CHECK(hipModuleLaunchKernel(kernel->function, grid[0], grid[1], grid[2], block[0], block[1], block[2],
                                       dyn_lds_bytes, dev->stream, nullptr, config));
