@@ -287,6 +287,20 @@ def build_workloads(w, dev, seeded, which, with_cpu=False):
         del hbm
         out["c5_mlp"] = Workload("config5c: GEMM f16 [2048x4096]x[4096x11008]", [[am.mat_mul(bm)]], 184683593728, "TFLOP/s",
                                  F16_MFMA_PEAK_TFLOPS, "f16", cpu=mlp_cpu)
+    if "attn" in which:
+        # batched products of attention shape (no BASELINE configuration; batched mat_mul is the reference's
+        # src/matmul.rs with leading dimensions): scores = q . k^T with k^T a transposed view, then p . v.  Both are
+        # bound by the [32,2048,2048] matrix they write or read, so they are priced against HBM.
+        F16 = np.float16
+        q = T.new(dev, seeded(6, 0, (32, 2048, 128), "normal", dtype=F16, std=0.1))
+        kk = T.new(dev, seeded(6, 1, (32, 2048, 128), "normal", dtype=F16, std=0.1))
+        v = T.new(dev, seeded(6, 2, (32, 2048, 128), "normal", dtype=F16, std=0.1))
+        pp = [T.new(dev, seeded(6, 3 + r, (32, 2048, 2048), "uniform", dtype=F16)) for r in range(2)]
+        small, big = 32 * 2048 * 128 * 2, 32 * 2048 * 2048 * 2
+        out["attn_qk"] = Workload("attention scores: q.k^T, f16 [32,2048,128]x[32,128,2048]", [[q.mat_mul(kk.transpose(1, 2))]],
+                                  2 * small + big, "GB/s", HBM_PEAK_GBS, "f16")
+        out["attn_pv"] = Workload("attention output: p.v, f16 [32,2048,2048]x[32,2048,128]", [[p_.mat_mul(v)] for p_ in pp],
+                                  big + 2 * small, "GB/s", HBM_PEAK_GBS, "f16")
     if "long" in which:
         # rows longer than a block's registers (no BASELINE configuration; the reference's reduce takes any length)
         xs = [T.new(dev, seeded(4, 40 + r, (256, 262144), "normal")) for r in range(2)]
@@ -385,7 +399,7 @@ def cpu_baseline(wl):
                       "oracle/port.c with OpenMP"}
 
 
-GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16", "long")
+GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16", "long", "attn")
 
 
 def plan_only(w):
@@ -612,7 +626,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="only the headline configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
-    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16,long for the detail table")
+    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16,long,attn for the detail table")
     ap.add_argument("--plan-only", action="store_true",
                     help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
     ap.add_argument("--profile", default="", help="run one workload only (copy, c1, c2a, c2b, c3, c4_rmsnorm, c4_rope, c4_softmax, "

@@ -817,7 +817,12 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 # a batch of one with a long K: few tiles, so K is cut into slices (256 x 256 and 128 x 128 tiles); the
                 # leading dimensions of size 1 must survive the fold of the slices
                 ((1,), 256, 256, 4096, False), ((1, 1), 256, 512, 2048, True), ((1,), 128, 384, 4096, False),
-                ((1, 1), 100, 136, 1024, False)]
+                ((1, 1), 100, 136, 1024, False),
+                # one column of 128-wide tiles over a long K (attention probabilities against values): every workgroup
+                # starts its walk over K at a different tile and wraps around; K with a partial last tile, B^T, edge columns
+                ((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False)]
+ROTATED = {((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False),
+           ((8,), 512, 128, 512, False)}
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -843,7 +848,10 @@ def test_batched_mat_mul(gpu, lead, m, n, k, bt, dtype, tol):
         gemm_check(got[idx], a[idx], np.ascontiguousarray(dense_b[idx]), tol)
     assert len([kk for kk in prod.kernels() if kk.kind == "gemm"]) == 1
     # and the same numbers as one product at a time (bit for bit when both take the same kernel with the same K slices)
-    if not bt and "skinny" not in prod.kernels()[0].detail:
+    gemm_of = lambda t: [kk for kk in t.kernels() if kk.kind == "gemm"][0].detail  # noqa: E731
+    if (lead, m, n, k, bt) in ROTATED and dtype == np.float16:
+        assert "K start rotated" in gemm_of(prod), gemm_of(prod)
+    if not bt and "skinny" not in prod.kernels()[0].detail and "slices" not in gemm_of(one):
         assert np.array_equal(alone, got[first])
     else:
         gemm_check(alone, a[first], np.ascontiguousarray(dense_b[first]), tol)

@@ -367,15 +367,19 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     if (nmain == 0 || ntail * 2 > cus) ntail = 0;
   }
   const bool tail = ntail > 0;
+  // one column of 128-wide tiles over a long K, B small enough to stay in L2: the workgroups share no rows of A and
+  // start their walk over K at different tiles (kernels/gemm_f16_t128.hip.inc, WKF_ROTK)
+  const bool rotk = t128 && !split && N <= 128 && K >= 512 && K * N * dtype_size(a.dtype) <= (size_t(1) << 20);
   TensorData out = split ? alloc(slices_shape(slices), DType::F32, false) : alloc(out_shape, a.dtype, false);
   std::string sig = t128 ? std::string("gemm|gfx950|f16|mfma32x32x16|128x128x64|w2x2|edge") : gemm_signature(kind, a.dtype);
   if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
   if (bt) sig += "|bt";
+  if (rotk) sig += "|rotk";
   if (tail) sig += "|last round in half tiles";
   wkf_kernel* k = kernel(sig, [&] {
     if (tail) return std::string(kGemmF16Tail);
     std::string src = bt ? "#define WKF_BT 1\n" : "";
-    if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + kGemmF16T128;
+    if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (rotk ? "#define WKF_ROTK 1\n" : "") + kGemmF16T128;
     if (!split) return src + gemm_source(kind, a.dtype);
     const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
     return src + "#define WKF_SPLITK 1\n" + gemm_source(base, a.dtype);
@@ -415,6 +419,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : t128 ? " mfma 128x128 tiles" : " mfma 256x256 tiles");
   if (!t128 && (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge)) d << " edge";
   if (bt) d << " B^T";
+  if (rotk) d << " K start rotated";
   if (split) d << " slices=" << slices;
   if (tail) d << ", last round: " << ntail << " tiles as " << 2 * ntail << " halves of 128 rows";
   if (batch > 1) d << " batch=" << batch;
