@@ -477,7 +477,8 @@ def test_batched_mat_mul_is_one_launch(wkf, planner):
     v = _x(wkf, planner, (8, 512, 128), np.float16, seed=2)
     out = scores.softmax_last_dim().mat_mul(v)
     assert out.shape() == (8, 512, 128) and _kinds(out) == ["gemm", "row", "gemm"]
-    assert out.kernels()[2].detail.endswith("128x128 tiles batch=8")    # n = 128: the small tile, nothing wasted
+    # n = 128: the small tile, nothing wasted; one column of tiles over K = 512: every workgroup starts at its own K tile
+    assert out.kernels()[2].detail.endswith("128x128 tiles K start rotated batch=8") and out.kernels()[2].signature.endswith("|rotk")
     r4 = _x(wkf, planner, (2, 3, 17, 33), np.float32).mat_mul(_x(wkf, planner, (2, 3, 33, 5), np.float32, seed=1))
     assert r4.shape() == (2, 3, 17, 5) and _kinds(r4) == ["gemm"] and r4.kernels()[0].detail.endswith("generic batch=6")
     # decode: one query row per head streams k and v once (the bandwidth kernels), one fold for all heads
