@@ -817,7 +817,7 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 # a batch of one with a long K: few tiles, so K is cut into slices (256 x 256 and 128 x 128 tiles); the
                 # leading dimensions of size 1 must survive the fold of the slices
                 ((1,), 256, 256, 4096, False), ((1, 1), 256, 512, 2048, True), ((1,), 128, 384, 4096, False),
-                ((1, 1), 100, 136, 1024, False),
+                ((1, 1), 100, 136, 1024, False), ((1,), 100, 102, 2048, True), ((1,), 120, 100, 1024, True),
                 # one column of 128-wide tiles over a long K (attention probabilities against values): every workgroup
                 # starts its walk over K at a different tile and wraps around; K with a partial last tile, B^T, edge columns
                 ((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False)]

@@ -338,8 +338,9 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   const size_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
   // ... and so do products that would waste half of every large tile (128 columns of attention values, say)
   const size_t pad256 = ((M + 255) / 256 * 256) * ((N + 255) / 256 * 256), pad128 = ((M + 127) / 128 * 128) * ((N + 127) / 128 * 128);
+  // (its loads take 32-bit byte offsets into a matrix: each operand matrix stays under 2 GiB)
   const bool t128 = mfma && a.dtype == DType::F16 && st_.fusion == FusionMode::Tree && st_.gemm_t128 &&
-                    (tiles256 * batch * 2 <= cus || pad128 * 20 <= pad256 * 11);
+                    (tiles256 * batch * 2 <= cus || pad128 * 20 <= pad256 * 11) && M * K < (size_t(1) << 30) && K * N < (size_t(1) << 30);
   const size_t tile = t128 ? 128 : 256;
   const size_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
   const size_t slots = t128 ? 2 * cus : cus;  // workgroups the chip holds at once
