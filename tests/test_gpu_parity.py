@@ -773,7 +773,10 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                (128, 128, 64), (129, 136, 64), (384, 640, 192), (200, 1000, 520), (511, 136, 2048), (33, 4096, 1024),
                # full tiles that leave a partly filled last round on 256 compute units (272, 300 and 257 tiles): in f16 the
                # tiles of that round run as two halves of 128 rows each
-               (4096, 4352, 512), (2560, 7680, 1024), (256, 65792, 2048)]
+               (4096, 4352, 512), (2560, 7680, 1024), (256, 65792, 2048),
+               # the same with ragged edges (272 and 288 tiles): a last tile row that ends inside its upper half (the lower
+               # half tiles do nothing), one that ends inside its lower half, ragged columns, a K that is no multiple of 64
+               (3900, 4360, 136), (4000, 4104, 72), (4090, 4352, 200)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

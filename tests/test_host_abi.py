@@ -431,7 +431,9 @@ def test_mat_mul_kernel_choice(wkf, planner):
     assert detail(4096, 4096, 128, np.float16).endswith("mfma 256x256 tiles")
     assert detail(512, 256, 96, np.float32).endswith("mfma 256x256 tiles")
     # not a multiple of the tile but every row 16-byte aligned: the same MFMA kernel with edge handling
-    assert detail(4000, 4104, 72, np.float16).endswith("mfma 256x256 tiles edge")
+    assert detail(4000, 4000, 72, np.float16).endswith("mfma 256x256 tiles edge")
+    # ... and a partly filled last round of it runs in half tiles like that of a full shape (16 x 17 tiles)
+    assert detail(4000, 4104, 72, np.float16).endswith("mfma 256x256 tiles edge, last round: 16 tiles as 32 halves of 128 rows")
     assert detail(300, 260, 68, np.float32).endswith("mfma 256x256 tiles edge")
     # f16 products whose large tiles would fill at most half of the chip take 128 x 128 tiles, two workgroups per compute unit
     assert detail(512, 256, 128, np.float16).endswith("mfma 128x128 tiles")
@@ -610,13 +612,15 @@ def test_gemm_kernels_use_no_scratch_memory(tmp_path):
         "    for bt in (False, True):\n"
         "        mm(4096, 4096, 128, dt, bt)    # full 256 x 256 tiles\n"
         "        mm(4096, 4352, 128, dt, bt)    # 272 tiles: the last round in half tiles (f16)\n"
-        "        mm(4000, 4104, 136, dt, bt)    # 256 x 256 tiles with ragged edges\n"
+        "        mm(4000, 4104, 136, dt, bt)    # 256 x 256 tiles with ragged edges (f16, B as it lies: the last round in half tiles)\n"
+        "        mm(4000, 4000, 136, dt, bt)    # ... in whole tiles\n"
         "        mm(512, 512, 256, dt, bt)      # few tiles\n"
         "        mm(300, 264, 2048, dt, bt)     # few ragged tiles, K in slices\n"
         "        mm(256, 256, 4096, dt, bt)     # K in slices\n"
         "        mm(128, 384, 4096, dt, bt)     # 128 x 128 tiles (f16), K in slices\n"
         "        mm(512, 1024, 512, dt, bt)     # 128 x 128 tiles (f16)\n"
         "        mm(1, 1024, 512, dt, bt); mm(8, 520, 1000, dt, bt); mm(20, 264, 4096, dt, bt)  # decode sizes\n"
+        "    mm(4000, 4001, 136, dt, True)      # rows of C off the 16-byte grid: the ragged kernel that addresses with pointers\n"
         "    mm(3, 5, 7, dt)                    # the generic kernel\n"
         "    mm(64, 64, 32, dt, lead=(3,))\n"
     )

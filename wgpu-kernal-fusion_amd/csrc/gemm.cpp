@@ -362,7 +362,8 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // of 128 rows each by twice as many workgroups, so that round fills twice as many compute units and takes about
   // half as long (kernels/gemm_f16_tail.hip.inc).
   size_t ntail = 0, nmain = 0;
-  if (kind == GemmKind::MfmaF16 && !bt && !t128 && !split && batch == 1 && st_.fusion == FusionMode::Tree && st_.gemm_tail) {
+  const bool tail_ragged = kind == GemmKind::MfmaF16Edge && K <= (size_t(1) << 21) && N <= (size_t(1) << 22) && N % 8 == 0;
+  if ((kind == GemmKind::MfmaF16 || tail_ragged) && !bt && !t128 && !split && batch == 1 && st_.fusion == FusionMode::Tree && st_.gemm_tail) {
     nmain = tiles / cus * cus;
     ntail = tiles - nmain;
     if (nmain == 0 || ntail * 2 > cus) ntail = 0;
@@ -373,14 +374,21 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   const bool rotk = t128 && !split && N <= 128 && K >= 512 && K * N * dtype_size(a.dtype) <= (size_t(1) << 20);
   TensorData out = split ? alloc(slices_shape(slices), DType::F32, false) : alloc(out_shape, a.dtype, false);
   std::string sig = t128 ? std::string("gemm|gfx950|f16|mfma32x32x16|128x128x64|w2x2|edge") : gemm_signature(kind, a.dtype);
+  // ragged f16 shapes (and K slices) on the large tile: buffer loads that read zeros past the edges, unless an offset
+  // inside a tile could pass 32 bits or rows of C do not start 16-byte aligned; those keep 64-bit pointers
+  const bool f16_large = !t128 && (kind == GemmKind::MfmaF16 || kind == GemmKind::MfmaF16Edge);
+  const bool ragged16 = f16_large && (split || kind == GemmKind::MfmaF16Edge);
+  const bool edge_ptr = ragged16 && !(K <= (size_t(1) << 21) && N <= (size_t(1) << 22) && N % 8 == 0);
   if (split) sig += sig.find("|edge") == std::string::npos ? "|edge|splitk" : "|splitk";
+  if (edge_ptr) sig += "|ptr";
   if (bt) sig += "|bt";
   if (rotk) sig += "|rotk";
-  if (tail) sig += "|last round in half tiles";
+  if (tail) sig += "|last round in half tiles";  // (a ragged shape keeps "|edge" in front of it)
   wkf_kernel* k = kernel(sig, [&] {
-    if (tail) return std::string(kGemmF16Tail);
+    if (tail) return std::string(tail_ragged ? "#define WKF_EDGEBUF 1\n" : "") + kGemmF16Tail;
     std::string src = bt ? "#define WKF_BT 1\n" : "";
     if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (rotk ? "#define WKF_ROTK 1\n" : "") + kGemmF16T128;
+    if (ragged16) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (edge_ptr ? "#define WKF_EDGE 1\n" : "#define WKF_EDGEBUF 1\n") + kGemmF16;
     if (!split) return src + gemm_source(kind, a.dtype);
     const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
     return src + "#define WKF_SPLITK 1\n" + gemm_source(base, a.dtype);
