@@ -104,7 +104,9 @@ int wkf_module_stats(wkf_device* dev, uint64_t* compiled, uint64_t* disk_hits, u
 /* Replaces begin_compute_pass / set_pipeline / set_bind_group /
  * dispatch_workgroups, src/kernel.rs:375-384.  `args` is the packed kernel
  * argument block (it also replaces the per-tensor uniform buffers of
- * src/kernel.rs:274-361).  hipModuleLaunchKernel on the device stream; when
+ * src/kernel.rs:274-361), laid out as the kernel's argument struct including
+ * its tail padding: `arg_bytes` is a multiple of 8 (anything else is refused).
+ * hipModuleLaunchKernel on the device stream; when
  * `timer` is non-NULL the launch carries the timer's two events in the dispatch
  * itself (hipExtModuleLaunchKernel): they take the kernel's own begin and end
  * timestamps, as the reference's timestamp queries around a compute pass do

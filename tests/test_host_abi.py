@@ -108,6 +108,15 @@ def test_misuse_returns_status_codes(wkf, planner):
         T.new(planner, [[1.0, 2.0], [3.0]])  # ragged input: the reference panics in IntoTensor
     with pytest.raises(wkf.WkfError):
         wkf.Device.new(99)
+    # level 0: an argument block cut short of its tail padding would reach the kernel without its last member
+    lib = wkf.load()
+    k = ctypes.c_void_p()
+    src = b'struct Args { float* p; unsigned n; }; extern "C" __global__ void k0(const Args a) { if (a.n) a.p[0] = 1.0f; }'
+    assert lib.wkf_module_get(planner._h, b"test|unpadded args", src, b"k0", ctypes.byref(k)) == 0, lib.wkf_last_error()
+    one = (ctypes.c_uint32 * 3)(1, 1, 1)
+    assert lib.wkf_launch(planner._h, k, one, one, 0, bytes(12), 12, None) == 3
+    assert b"multiple of 8" in lib.wkf_last_error()
+    assert lib.wkf_launch(planner._h, k, one, one, 0, bytes(16), 16, None) == 0
 
 
 def test_layout_view_algebra(wkf, planner):

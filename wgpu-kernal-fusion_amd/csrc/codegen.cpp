@@ -263,13 +263,114 @@ std::string map_signature(const MapSpec& s) {
   if (s.tile_dim >= 0) {
     o << "|tile" << s.tile_dim << ':';
     for (size_t k = 0; k < s.in.size(); k++) o << (s.crossed[k] ? 'x' : '-');
+    if (s.tile_vec > 1) o << "|tv" << s.tile_vec;
   }
   return o.str();
 }
 
 namespace {
 // out = expr(inputs) where some inputs run along `tile_dim` and the output along the last dimension.
+// The same with four elements per global access.  A thread is lane q = t % 16 of row r = t / 16: sixteen lanes cover the
+// 64 elements of a tile row along the operand's unit-stride dimension, a pass covers 16 rows, four passes the tile.
+// The LDS tile is [b][a] with an odd pitch in 4-byte words, so the four scalar writes of a vector read along a and
+// the four scalar reads of a vector written along b are both free of bank conflicts.
+std::string map_tiled_vec_source(const MapSpec& s) {
+  const int N = int(s.in.size()) + 1;
+  const int R = s.rank, TA = s.tile_dim, TB = s.rank - 1;
+  const int NC = s.prog.consts.empty() ? 1 : int(s.prog.consts.size());
+  std::ostringstream o;
+  o << kPrelude;
+  if (uses_math(s.prog, s.math)) o << kMath;
+  if (uses_round_h(s.prog, s.math)) o << kRoundH;
+  o << "struct Args { void* p[" << N << "]; u32 nwork; u32 shape[" << R << "]; u32 off[" << N << "]; u32 stride[" << N
+    << "][" << R << "]; float c[" << NC << "]; };\n";
+  std::vector<DType> types;
+  for (const auto& i : s.in) types.push_back(i.dtype);
+  emit_program(o, s.prog, "wkf_expr", types, s.math);
+  const bool trig = uses_trig(s.prog, s.math);
+  auto dt = [&](int k) { return k < N - 1 ? s.in[k].dtype : s.out.dtype; };
+  auto ptr = [&](int k) {
+    return std::string("((") + (k < N - 1 ? "const " : "") + ctype(dt(k)) + "*)a.p[" + std::to_string(k) + "])";
+  };
+  o << "extern \"C\" __global__ void __launch_bounds__(" << kMapBlock << ") WKF_ENTRY(const Args a) {\n";
+  for (int k = 0; k < N - 1; k++)
+    if (s.crossed[k])
+      o << "  __shared__ " << ctype(dt(k)) << " tile" << k << "[" << kMapTile << "][" << kMapTile + (dtype_size(dt(k)) == 2 ? 2 : 1) << "];\n";
+  o << "  const u32 q = threadIdx.x & 15u, r = threadIdx.x >> 4;\n";
+  o << "  const u32 A = a.shape[" << TA << "], B = a.shape[" << TB << "];\n";
+  o << "  const u32 tiles_a = (A + 63u) / 64u, tiles_b = (B + 63u) / 64u;\n";
+  // Tiles are walked along b, each row of tiles starting one tile further on (a diagonal order): workgroups that run
+  // at the same time then touch rows of the crossed operands whose distance is not a fixed multiple of 64 rows
+  // (measured on an f32 [8192,8192] transposing copy: 3959 -> 4582 GB/s, with the non-temporal bits 5082).
+  o << "  u32 rem = blockIdx.x;\n";
+  o << "  const u32 tb_ = rem % tiles_b; rem /= tiles_b;\n";
+  o << "  const u32 ta_ = rem % tiles_a; rem /= tiles_a;\n";
+  o << "  const u32 b0 = ((tb_ + ta_) % tiles_b) * 64u, a0 = ta_ * 64u;\n";
+  std::vector<int> others;
+  for (int d = R - 2; d >= 0; d--)
+    if (d != TA) others.push_back(d);
+  for (size_t i = 0; i < others.size(); i++) {
+    const int d = others[i];
+    if (i + 1 < others.size()) o << "  const u32 i" << d << " = rem % a.shape[" << d << "]; rem /= a.shape[" << d << "];\n";
+    else o << "  const u32 i" << d << " = rem;\n";
+  }
+  for (int k = 0; k < N; k++) {
+    o << "  const u32 base" << k << " = a.off[" << k << "]";
+    for (int d : others) o << " + i" << d << " * a.stride[" << k << "][" << d << "]";
+    o << ";\n";
+  }
+  // phase 1: crossed inputs, a vector along tile_dim per lane (indices clamped: every load is unconditional; A and B
+  // are multiples of 4, so a vector lies inside or outside as a whole)
+  for (int k = 0; k < N - 1; k++) {
+    if (!s.crossed[k]) continue;
+    std::string vt = vtype(dt(k), 4);
+    o << "  {\n    " << vt << " v[4];\n";
+    o << "    const u32 aa = min(a0 + q * 4u, A - 4u);\n";
+    o << "#pragma unroll\n    for (int j = 0; j < 4; j++) {\n";
+    o << "      const u32 bb = min(b0 + r + 16u * j, B - 1u);\n";
+    o << "      v[j] = " << (s.nontemporal ? "__builtin_nontemporal_load(" : "*(") << "(const " << vt << "*)(" << ptr(k) << " + (base" << k
+      << " + aa + bb * a.stride[" << k << "][" << TB << "])));\n    }\n";
+    o << "#pragma unroll\n    for (int j = 0; j < 4; j++)\n#pragma unroll\n      for (int e = 0; e < 4; e++) tile" << k
+      << "[r + 16u * j][q * 4u + e] = v[j][e];\n  }\n";
+  }
+  o << "  __syncthreads();\n";
+  // phase 2: a vector along the last dim per lane
+  o << "  const u32 bb = min(b0 + q * 4u, B - 4u);\n";
+  o << "  const bool b_live = b0 + q * 4u < B;\n";
+  std::string ovt = vtype(s.out.dtype, 4);
+  o << "#pragma unroll\n  for (int j = 0; j < 4; j++) {\n";
+  o << "    const u32 al = r + 16u * j, aa = a0 + al, ac = min(aa, A - 1u);\n";
+  for (int k = 0; k < N - 1; k++) {
+    if (s.crossed[k]) continue;
+    if (s.in[k].inner_stride == 1)
+      o << "    const " << vtype(dt(k), 4) << " s" << k << " = " << (s.nontemporal ? "__builtin_nontemporal_load(" : "*(") << "(const " << vtype(dt(k), 4)
+        << "*)(" << ptr(k) << " + (base" << k << " + ac * a.stride[" << k << "][" << TA << "] + bb)));\n";
+    else
+      o << "    const " << ctype(dt(k)) << " s" << k << " = " << ptr(k) << "[base" << k << " + ac * a.stride[" << k << "][" << TA << "]];\n";
+  }
+  o << "    " << ovt << " ov;\n";
+  for (int e = 0; e < 4; e++) {
+    std::ostringstream call;
+    for (int k = 0; k < N - 1; k++) {
+      if (s.crossed[k]) call << "tile" << k << "[q * 4u + " << e << "][al], ";
+      else if (s.in[k].inner_stride == 1) call << "s" << k << "[" << e << "], ";
+      else call << "s" << k << ", ";
+    }
+    o << "    {\n";
+    if (trig) o << "      bool far = false;\n";
+    o << "      " << ctype(s.out.dtype) << " v = wkf_expr(" << call.str() << "a.c" << (trig ? ", far" : "") << ");\n";
+    if (trig) o << "      if (__builtin_expect(far, 0)) v = wkf_expr_far(" << call.str() << const_args(s.prog, "a.c", 0, true) << ");\n";
+    o << "      ov[" << e << "] = v;\n    }\n";
+  }
+  o << "    if (b_live && aa < A) ";
+  if (s.nontemporal) o << "__builtin_nontemporal_store(ov, (" << ovt << "*)(" << ptr(N - 1) << " + (base" << N - 1 << " + aa * a.stride[" << N - 1 << "][" << TA << "] + bb)));\n";
+  else o << "*(" << ovt << "*)(" << ptr(N - 1) << " + (base" << N - 1 << " + aa * a.stride[" << N - 1 << "][" << TA << "] + bb)) = ov;\n";
+  o << "  }\n}\n";
+  return o.str();
+}
+
 std::string map_tiled_source(const MapSpec& s) {
+  if (s.tile_vec == 4) return map_tiled_vec_source(s);
   const int N = int(s.in.size()) + 1;
   const int R = s.rank, TA = s.tile_dim, TB = s.rank - 1;
   const int NC = s.prog.consts.empty() ? 1 : int(s.prog.consts.size());
@@ -295,9 +396,13 @@ std::string map_tiled_source(const MapSpec& s) {
   o << "  const u32 tx = threadIdx.x & 63u, ty = threadIdx.x >> 6;\n";
   o << "  const u32 A = a.shape[" << TA << "], B = a.shape[" << TB << "];\n";
   o << "  const u32 tiles_a = (A + 63u) / 64u, tiles_b = (B + 63u) / 64u;\n";
+  // Tiles are walked along b, each row of tiles starting one tile further on (a diagonal order): workgroups that run
+  // at the same time then touch rows of the crossed operands whose distance is not a fixed multiple of 64 rows
+  // (measured on an f32 [8192,8192] transposing copy: 3959 -> 4582 GB/s, with the non-temporal bits 5082).
   o << "  u32 rem = blockIdx.x;\n";
-  o << "  const u32 b0 = (rem % tiles_b) * 64u; rem /= tiles_b;\n";
-  o << "  const u32 a0 = (rem % tiles_a) * 64u; rem /= tiles_a;\n";
+  o << "  const u32 tb_ = rem % tiles_b; rem /= tiles_b;\n";
+  o << "  const u32 ta_ = rem % tiles_a; rem /= tiles_a;\n";
+  o << "  const u32 b0 = ((tb_ + ta_) % tiles_b) * 64u, a0 = ta_ * 64u;\n";
   std::vector<int> others;
   for (int d = R - 2; d >= 0; d--)
     if (d != TA) others.push_back(d);

@@ -40,6 +40,10 @@ struct MapSpec {
   // 64 x 64 tile of (tile_dim, last dim): crossed inputs are read along tile_dim into LDS and read back
   // along the last dim, so global loads and stores are both coalesced.  vec is 1.
   int tile_dim = -1;
+  // tile_vec == 4: every operand is read and written four elements at a time along its unit-stride dimension (both
+  // tile extents are multiples of 4, every other stride and every offset too); non-crossed inputs then have
+  // inner_stride 1 (a vector per lane) or 0 (one value per tile row)
+  int tile_vec = 1;
   std::vector<bool> crossed;         // per input; used when tile_dim >= 0
   int rank;                          // rank of the coalesced iteration space (1..kMaxRank)
   int vec;                           // elements per work item: 1, 2, 4 or 8

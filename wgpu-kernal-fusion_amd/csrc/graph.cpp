@@ -1051,11 +1051,29 @@ void Resolver::launch_map_tiled(MapSpec& spec, const Space& sp, const std::vecto
   auto td_of = [&](size_t k) -> const TensorData& { return k < in.size() ? in[k] : out; };
   spec.unroll = 1;
   spec.nontemporal = false;
+  // four elements per access when every operand allows it: unit stride along its own dimension of the tile (or, for an
+  // input that does not cross, none along the last one), everything else a multiple of four elements
+  bool vec4 = st_.map_tile_vec && sp.shape[ta] % 4 == 0 && sp.shape[R - 1] % 4 == 0;
+  for (size_t k = 0; k < N && vec4; k++) {
+    const bool crossed = k < in.size() && spec.crossed[k];
+    const size_t own = crossed ? ta : R - 1;
+    const size_t s_own = sp.strides[k][own];
+    if (!(s_own == 1 || (!crossed && k < in.size() && s_own == 0))) vec4 = false;
+    for (size_t d = 0; d < R; d++)
+      if (d != own && sp.strides[k][d] % 4) vec4 = false;
+    if (td_of(k).layout.offset % 4) vec4 = false;
+  }
+  spec.tile_vec = vec4 ? 4 : 1;
+  {
+    size_t bytes = 0;
+    for (size_t k = 0; k < N; k++) bytes += out.layout.numel() * dtype_size(td_of(k).dtype);
+    spec.nontemporal = vec4 && bytes >= st_.nontemporal_bytes;
+  }
   for (size_t k = 0; k < N; k++) {
     MapOperandSpec os;
     os.dtype = td_of(k).dtype;
     os.linear = false;
-    os.inner_stride = -1;
+    os.inner_stride = vec4 && k < in.size() && !spec.crossed[k] ? int(sp.strides[k][R - 1]) : -1;
     if (k < in.size()) spec.in.push_back(os);
     else spec.out = os;
   }
@@ -1085,7 +1103,7 @@ void Resolver::launch_map_tiled(MapSpec& spec, const Space& sp, const std::vecto
   r.grid[0] = to_u32(blocks, "grid");
   r.block[0] = kMapBlock;
   std::ostringstream d;
-  d << "shape=" << dims(sp.shape) << " tiled dim=" << ta << " operands=" << N << (in_place ? " in_place" : "");
+  d << "shape=" << dims(sp.shape) << " tiled dim=" << ta << " operands=" << N << (vec4 ? " vec=4" : "") << (in_place ? " in_place" : "");
   r.detail = d.str();
   r.in_place = in_place;
   record(std::move(r), k, map_pack_args(spec, args));

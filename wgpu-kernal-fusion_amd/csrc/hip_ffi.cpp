@@ -570,6 +570,9 @@ int wkf_launch(wkf_device* dev, wkf_kernel* kernel, const uint32_t grid[3], cons
   uint64_t threads = uint64_t(block[0]) * block[1] * block[2];
   if (!threads || threads > 1024 || !grid[0] || !grid[1] || !grid[2] || grid[1] > 65535 || grid[2] > 65535)
     return fail(WKF_ERR_INVALID_ARG, "wkf_launch: bad launch geometry");
+  // An argument block that holds a pointer is 8-byte aligned and so is its size; a block cut short of its tail padding
+  // reaches the kernel without its last member.
+  if (arg_bytes % 8 != 0) return fail(WKF_ERR_INVALID_ARG, "wkf_launch: the argument block must be padded to a multiple of 8 bytes");
   if (dev->planner) return WKF_OK;  // plan-only: nothing runs
   if (!kernel->function) return fail(WKF_ERR_INVALID_ARG, "wkf_launch: kernel has no loaded function");
   std::lock_guard<std::recursive_mutex> lock(dev->mu);
