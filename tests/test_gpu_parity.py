@@ -227,10 +227,16 @@ def test_transposed_operands_with_aligned_shapes(gpu, dtype):
                 ta.slice([(8, 296), (16, 504)]).transpose(0, 1) * tb.slice([(16, 504), (8, 296)]),
                 ta.transpose(0, 1).exp() + tb]
 
+    ts = progs(api.tensor(a), api.tensor(b), api.tensor(c), api.tensor(r))
+    alone = [hip_values(t) for t in ts]
+    # every one of them moves four elements per access on both sides of the tile
+    for i, t in enumerate(ts):
+        assert any(k.kind == "map" and "tiled" in k.detail and "vec=4" in k.detail for k in t.kernels()), (i, [k.detail for k in t.kernels()])
     got = hip_values_many(progs(api.tensor(a), api.tensor(b), api.tensor(c), api.tensor(r)))
     want = progs(OTensor(a), OTensor(b), OTensor(c), OTensor(r))
     for i, (g, w) in enumerate(zip(got, want)):
         assert_ulp(g, w.to_numpy(), 0, f"program {i}")
+        assert np.array_equal(alone[i], g), i
 
 
 def test_same_results_under_both_fusion_modes(gpu):

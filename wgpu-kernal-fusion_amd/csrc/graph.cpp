@@ -1058,7 +1058,8 @@ void Resolver::launch_map_tiled(MapSpec& spec, const Space& sp, const std::vecto
     const bool crossed = k < in.size() && spec.crossed[k];
     const size_t own = crossed ? ta : R - 1;
     const size_t s_own = sp.strides[k][own];
-    if (!(s_own == 1 || (!crossed && k < in.size() && s_own == 0))) vec4 = false;
+    if (!crossed && k < in.size() && s_own == 0) continue;  // one value per tile row: a scalar load, nothing to align
+    if (s_own != 1) vec4 = false;
     for (size_t d = 0; d < R; d++)
       if (d != own && sp.strides[k][d] % 4) vec4 = false;
     if (td_of(k).layout.offset % 4) vec4 = false;
