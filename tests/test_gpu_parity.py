@@ -782,7 +782,9 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                (4096, 4352, 512), (2560, 7680, 1024), (256, 65792, 2048),
                # the same with ragged edges (272 and 288 tiles): a last tile row that ends inside its upper half (the lower
                # half tiles do nothing), one that ends inside its lower half, ragged columns, a K that is no multiple of 64
-               (3900, 4360, 136), (4000, 4104, 72), (4090, 4352, 200)]
+               (3900, 4360, 136), (4000, 4104, 72), (4090, 4352, 200),
+               # 1024 full tiles over K = 64 and K = 128: the kernel that keeps a tile's whole K in the LDS
+               (8192, 8192, 64), (4096, 16384, 128)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -830,6 +832,9 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 # one column of 128-wide tiles over a long K (attention probabilities against values): every workgroup
                 # starts its walk over K at a different tile and wraps around; K with a partial last tile, B^T, edge columns
                 ((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False)]
+# many full tiles over K = 64 or 128: one workgroup per compute unit walks the tiles of the whole batch
+BATCH_SHAPES += [((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True)]
+WHOLE_K = {((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True)}
 ROTATED = {((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False),
            ((8,), 512, 128, 512, False)}
 
@@ -858,6 +863,8 @@ def test_batched_mat_mul(gpu, lead, m, n, k, bt, dtype, tol):
     assert len([kk for kk in prod.kernels() if kk.kind == "gemm"]) == 1
     # and the same numbers as one product at a time (bit for bit when both take the same kernel with the same K slices)
     gemm_of = lambda t: [kk for kk in t.kernels() if kk.kind == "gemm"][0].detail  # noqa: E731
+    if (lead, m, n, k, bt) in WHOLE_K and dtype == np.float16:
+        assert "whole K in LDS" in gemm_of(prod), gemm_of(prod)
     if (lead, m, n, k, bt) in ROTATED and dtype == np.float16:
         assert "K start rotated" in gemm_of(prod), gemm_of(prod)
     if not bt and "skinny" not in prod.kernels()[0].detail and "slices" not in gemm_of(one):

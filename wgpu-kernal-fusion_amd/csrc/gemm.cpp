@@ -32,6 +32,9 @@ const char* const kGemmF16T128 =
 const char* const kGemmF16Tail =
 #include "kernels/gemm_f16_tail.hip.inc"
     ;
+const char* const kGemmF16ShortK =
+#include "kernels/gemm_f16_shortk.hip.inc"
+    ;
 // most rows of A the lane-per-column bandwidth kernel takes (accumulators: rows x 8 per lane for f16, rows x 4 for f32;
 // f32 has no MFMA decode kernel for a row-major B, and a 256-row MFMA tile for 32 rows of f32 is 3 times slower still)
 constexpr size_t kSkinnyRowsF16 = 16, kSkinnyRowsF32 = 32;
@@ -369,6 +372,11 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     if (nmain == 0 || ntail * 2 > cus) ntail = 0;
   }
   const bool tail = ntail > 0;
+  // Many full tiles over K = 64 or 128 (attention scores, a low-rank update): what bounds them is the stores of C.  One
+  // workgroup per compute unit walks the tiles of the whole batch with the next tile's operands in flight under the
+  // current tile's MFMAs and stores (kernels/gemm_f16_shortk.hip.inc).
+  const bool shortk = kind == GemmKind::MfmaF16 && !t128 && !split && !tail && st_.fusion == FusionMode::Tree && st_.gemm_shortk &&
+                      (K == 64 || K == 128) && tiles * batch >= 4 * cus && cus % 8 == 0 && tiles * batch <= 0xffffffffull;
   // one column of 128-wide tiles over a long K, B small enough to stay in L2: the workgroups share no rows of A and
   // start their walk over K at different tiles (kernels/gemm_f16_t128.hip.inc, WKF_ROTK)
   const bool rotk = t128 && !split && N <= 128 && K >= 512 && K * N * dtype_size(a.dtype) <= (size_t(1) << 20);
@@ -383,11 +391,13 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (edge_ptr) sig += "|ptr";
   if (bt) sig += "|bt";
   if (rotk) sig += "|rotk";
+  if (shortk) sig += K == 64 ? "|whole K in LDS|nt1" : "|whole K in LDS|nt2";
   if (tail) sig += "|last round in half tiles";  // (a ragged shape keeps "|edge" in front of it)
   wkf_kernel* k = kernel(sig, [&] {
     if (tail) return std::string(tail_ragged ? "#define WKF_EDGEBUF 1\n" : "") + kGemmF16Tail;
     std::string src = bt ? "#define WKF_BT 1\n" : "";
     if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (rotk ? "#define WKF_ROTK 1\n" : "") + kGemmF16T128;
+    if (shortk) return src + (K == 64 ? "#define WKF_NT 1\n" : "#define WKF_NT 2\n") + kGemmF16ShortK;
     if (ragged16) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (edge_ptr ? "#define WKF_EDGE 1\n" : "#define WKF_EDGEBUF 1\n") + kGemmF16;
     if (!split) return src + gemm_source(kind, a.dtype);
     const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
@@ -401,6 +411,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     uint32_t m, n, k, kchunk;
   } args = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(out.buffer.get()),
             uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(kchunk)};
+  if (shortk) args.kchunk = uint32_t(batch);  // the kernel walks the tiles of every matrix itself
   std::vector<unsigned char> bytes(sizeof(args));
   memcpy(bytes.data(), &args, sizeof(args));
   if (tail) {
@@ -420,15 +431,16 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     if (r.grid[1] > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many rows for the generic kernel");
   } else {
     if (tiles > 0x7fffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
-    r.grid[0] = uint32_t(tail ? nmain + 2 * ntail : tiles);
+    r.grid[0] = uint32_t(shortk ? cus : tail ? nmain + 2 * ntail : tiles);
     r.grid[1] = uint32_t(slices);
   }
-  r.grid[2] = uint32_t(batch);
+  r.grid[2] = uint32_t(shortk ? 1 : batch);
   std::ostringstream d;
   d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : t128 ? " mfma 128x128 tiles" : " mfma 256x256 tiles");
   if (!t128 && (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge)) d << " edge";
   if (bt) d << " B^T";
   if (rotk) d << " K start rotated";
+  if (shortk) d << ", whole K in LDS, one workgroup per compute unit walks the tiles";
   if (split) d << " slices=" << slices;
   if (tail) d << ", last round: " << ntail << " tiles as " << 2 * ntail << " halves of 128 rows";
   if (batch > 1) d << " batch=" << batch;

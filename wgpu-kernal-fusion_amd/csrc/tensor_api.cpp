@@ -115,6 +115,7 @@ Settings settings_for(wkf_device* dev) {
       if (v >= 1 && v <= 1024 && (v & (v - 1)) == 0) st.row_threads = v;
     }
     if (const char* u = getenv("WKF_GEMM_T128")) st.gemm_t128 = atoi(u) != 0;
+    if (const char* u = getenv("WKF_GEMM_SHORTK")) st.gemm_shortk = atoi(u) != 0;
     if (const char* u = getenv("WKF_MAP_TILE_VEC")) st.map_tile_vec = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_TAIL")) st.gemm_tail = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_SPLIT")) st.row_split = atoi(u) != 0;
