@@ -336,14 +336,18 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (wkf_device_props(dev_, &props) != WKF_OK) throw Error(WKF_ERR_HIP, wkf_last_error());
   const size_t cus = size_t(std::max(1, props.compute_units));
   // f16 products whose 256 x 256 tiles would fill at most half of the chip take 128 x 128 tiles, two workgroups per
-  // compute unit ([512 x 4096] x [4096 x 11008]: 92 us against 109; with 172 of the large tiles, [1024 x ...], the large
-  // tile is the faster one again: 119 us against 159)
+  // compute unit ([512 x 4096] x [4096 x 11008]: 68 us against 109; with 172 of the large tiles, [1024 x ...], the large
+  // tile is the faster one again: 97 us against 114)
   const size_t tiles256 = ((M + 255) / 256) * ((N + 255) / 256);
   // ... and so do products that would waste half of every large tile (128 columns of attention values, say)
   const size_t pad256 = ((M + 255) / 256 * 256) * ((N + 255) / 256 * 256), pad128 = ((M + 127) / 128 * 128) * ((N + 127) / 128 * 128);
+  // ... but not a single product over a long K with 48 large tiles or more: cut into K slices those fill the chip, and
+  // over a long K the large tile's lower LDS traffic per flop outweighs the partial sums ([1280 x 11008] x [11008 x 4096]:
+  // 121 us in 3 slices against 174 on the small tile; at K = 4096 the small tile still wins: 54 against 61 for [1024 x ...])
+  const bool long_k_in_slices = batch == 1 && K >= 8192 && tiles256 >= 48;
   // (its loads take 32-bit byte offsets into a matrix: each operand matrix stays under 2 GiB)
   const bool t128 = mfma && a.dtype == DType::F16 && st_.fusion == FusionMode::Tree && st_.gemm_t128 &&
-                    (tiles256 * batch * 2 <= cus || pad128 * 20 <= pad256 * 11) && M * K < (size_t(1) << 30) && K * N < (size_t(1) << 30);
+                    ((tiles256 * batch * 2 <= cus && !long_k_in_slices) || pad128 * 20 <= pad256 * 11) && M * K < (size_t(1) << 30) && K * N < (size_t(1) << 30);
   const size_t tile = t128 ? 128 : 256;
   const size_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
   const size_t slots = t128 ? 2 * cus : cus;  // workgroups the chip holds at once
