@@ -87,13 +87,32 @@ def measure_kernels(dev, wl, steps, warmup):
         wl.step(i)
     dev.sync()
     samples, kinds, details = [], None, None
-    for i in range(steps):
+    # The next step is enqueued before the times of the step before it are read (a different input variant, so its
+    # kernel records are not the ones being read): reading a time waits for its kernel, and on some machines a GPU that
+    # waits for the host between two short kernels drops its clocks (seen: 30 us per launch read one by one against
+    # 23 us for a 128 MiB map kernel).  With a single variant the steps are read one by one.
+    ahead = len(wl.variants) >= 2
+
+    def read(outs):
+        nonlocal kinds, details
         ks = []
-        for t in wl.step(i):
+        for t in outs:
             ks += t.kernels()
         samples.append([k.elapsed_ns for k in ks])
         kinds = [k.kind for k in ks]
         details = [k.detail for k in ks]
+
+    before = None
+    for i in range(steps):
+        outs = wl.step(i)
+        if not ahead:
+            read(outs)
+            continue
+        if before is not None:
+            read(before)
+        before = outs
+    if before is not None:
+        read(before)
     arr = np.array(samples, dtype=np.float64) / 1e3  # [step][kernel] in us
     med, mn = np.median(arr, axis=0), arr.min(axis=0)
     total = arr.sum(axis=1)
