@@ -51,3 +51,34 @@ def test_inplace_reuse_never_touches_a_leaf(gpu, wkf):
             gpu.set_fusion(1)
         assert np.array_equal(got[1], (data + data) * data)
         assert np.array_equal(leaf.to_numpy(), data)
+
+
+def test_kernel_times_from_both_kinds_of_events(gpu):
+    # PerformanceQueries / all_timing_information (src/query.rs:50-126, src/tensor.rs:556-558): every launch reports a
+    # time, whether its two events ride in the dispatch (the default) or are recorded around it (WKF_TIMER_EVENTS=1,
+    # also the path of grids beyond 2^32 work-items); the second kind is read once per process, hence the child process
+    if gpu.is_planner:
+        from helpers import load_package
+        x = load_package().Tensor.new(gpu, np.ones((1024, 1024), dtype=np.float32))
+        ((x * 2.0) + 1.0).sum(1).materialize()  # the child's kernel goes into the cache
+        pytest.skip("plan-only device: nothing runs, nothing is timed")
+    import os
+    import subprocess
+    import sys
+    from helpers import ROOT
+    script = (
+        "import sys, numpy as np\n"
+        f"sys.path.insert(0, {os.path.join(ROOT, 'tests')!r})\n"
+        "from helpers import load_package\n"
+        "w = load_package(); dev = w.Device.new(0)\n"
+        "x = w.Tensor.new(dev, np.ones((1024, 1024), dtype=np.float32))\n"
+        "y = ((x * 2.0) + 1.0).sum(1)\n"
+        "assert np.array_equal(y.to_numpy(), np.full(1024, 3072.0, dtype=np.float32))\n"
+        "ks = y.kernels()\n"
+        "assert len(ks) == 1 and 500 < ks[0].elapsed_ns < 5_000_000, ks\n"
+        "print('timed', ks[0].elapsed_ns)\n"
+    )
+    for events in ("0", "1"):
+        env = dict(os.environ, WKF_TIMER_EVENTS=events)
+        out = subprocess.run([sys.executable, "-c", script], env=env, capture_output=True, text=True, timeout=110)
+        assert out.returncode == 0 and "timed" in out.stdout, (events, out.stdout, out.stderr[-2000:])
