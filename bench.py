@@ -320,6 +320,22 @@ def build_workloads(w, dev, seeded, which, with_cpu=False):
                                   2 * small + big, "GB/s", HBM_PEAK_GBS, "f16")
         out["attn_pv"] = Workload("attention output: p.v, f16 [32,2048,2048]x[32,2048,128]", [[p_.mat_mul(v)] for p_ in pp],
                                   big + 2 * small, "GB/s", HBM_PEAK_GBS, "f16")
+    if "more" in which:
+        # shapes off the BASELINE list that have kernels of their own: a transposed operand, a ragged product, a product
+        # of a few hundred rows against a wide weight
+        xt = [T.new(dev, seeded(7, r, (8192, 8192), "normal")) for r in range(3)]
+        out["more_transpose"] = Workload("transposed operand: x^T + 1, f32 [8192,8192]", [[x.transpose(0, 1) + 1.0] for x in xt],
+                                         2 * 8192 * 8192 * 4, "GB/s", HBM_PEAK_GBS)
+        del xt
+        F16 = np.float16
+        ar = T.new(dev, seeded(7, 4, (4000, 4096), "normal", dtype=F16, std=0.02))
+        br = T.new(dev, seeded(7, 5, (4096, 4096), "normal", dtype=F16, std=0.02))
+        out["more_gemm_ragged"] = Workload("ragged product: GEMM f16 [4000x4096]x[4096x4096]", [[ar.mat_mul(br)]], 2 * 4000 * 4096 * 4096,
+                                           "TFLOP/s", F16_MFMA_PEAK_TFLOPS, "f16")
+        am_ = T.new(dev, seeded(7, 6, (512, 4096), "normal", dtype=F16, std=0.02))
+        bm_ = T.new(dev, seeded(7, 7, (4096, 11008), "normal", dtype=F16, std=0.02))
+        out["more_gemm_mid"] = Workload("512 rows against a wide weight: GEMM f16 [512x4096]x[4096x11008]", [[am_.mat_mul(bm_)]],
+                                        2 * 512 * 4096 * 11008, "TFLOP/s", F16_MFMA_PEAK_TFLOPS, "f16")
     if "long" in which:
         # rows longer than a block's registers (no BASELINE configuration; the reference's reduce takes any length)
         xs = [T.new(dev, seeded(4, 40 + r, (256, 262144), "normal")) for r in range(2)]
@@ -418,7 +434,7 @@ def cpu_baseline(wl):
                       "oracle/port.c with OpenMP"}
 
 
-GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16", "long", "attn")
+GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16", "long", "attn", "more")
 
 
 def plan_only(w):
@@ -645,7 +661,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="only the headline configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
-    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16,long,attn for the detail table")
+    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16,long,attn,more for the detail table")
     ap.add_argument("--plan-only", action="store_true",
                     help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
     ap.add_argument("--profile", default="", help="run one workload only (copy, c1, c2a, c2b, c3, c4_rmsnorm, c4_rope, c4_softmax, "
