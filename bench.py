@@ -511,6 +511,33 @@ extern "C" __global__ void __launch_bounds__(256) wkf_mfma_only(const Args g) {
 }
 """
 
+MFMA_ONLY_F32_SRC = r"""
+// Yardstick: the MFMA work of the f32 256 x 256 x K tile kernel and nothing else: 256 v_mfma_f32_32x32x2_f32 per
+// wave and 32 columns of K, operands taken once from A and B (real data).
+typedef unsigned int u32;
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float acc16 __attribute__((ext_vector_type(16)));
+struct Args { const float* a; const float* b; float* c; u32 m, n, k, kchunk; };
+extern "C" __global__ void __launch_bounds__(256) wkf_mfma_only_f32(const Args g) {
+  const u32 tid = threadIdx.x;
+  f4 fa[4], fb[4];
+  for (int i = 0; i < 4; i++) fa[i] = *(const f4*)(g.a + (size_t(blockIdx.x) * 256 + tid) * 16 + i * 4);
+  for (int i = 0; i < 4; i++) fb[i] = *(const f4*)(g.b + (size_t(blockIdx.x) * 256 + tid) * 16 + i * 4);
+  acc16 acc[16];
+  for (int i = 0; i < 16; i++) acc[i] = (acc16)(0.0f);
+  for (u32 t = 0; t < g.k / 32; t++) {
+#pragma unroll
+    for (int r = 0; r < 16; r++)
+#pragma unroll
+      for (int i = 0; i < 16; i++)
+        acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[(i >> 2)][(r + i) & 3], fb[i & 3][r & 3], acc[i], 0, 0, 0);
+  }
+  float s = 0;
+  for (int i = 0; i < 16; i++) s += acc[i][0] + acc[i][7];
+  g.c[size_t(blockIdx.x) * 256 + tid] = s;
+}
+"""
+
 STREAM_SRC = r"""
 // Yardstick: plain streaming kernels over 1 GiB buffers (MODE 0 copy, 1 read-only, 2 write-only, 3 two reads and
 // one write: out = in + in2), U 16-byte accesses per lane and stream in flight, non-temporal bits on the loads
@@ -620,6 +647,21 @@ def yardsticks(w, dev, seeded, which, launches):
             for bf in (ba, bb, bc):
                 lib.wkf_buffer_release(bf)
         out["mfma_only_4096x4096x4096_equivalent"] = rows
+        # the same for the f32 kernel (v_mfma_f32_32x32x2_f32, nominal peak 157.3 TFLOP/s)
+        k32 = kernel("yardstick|mfma_only|f32 32x32x2", MFMA_ONLY_F32_SRC, "wkf_mfma_only_f32")
+        rows32 = []
+        for label, a, b in (("config-5 operands, N(0, 0.02)", seeded(5, 0, (4096, 4096), "normal", std=0.02),
+                             seeded(5, 1, (4096, 4096), "normal", std=0.02)),
+                            ("zeros", np.zeros((4096, 4096), np.float32), np.zeros((4096, 4096), np.float32))):
+            ba, bb, bc = dev_buf(a.nbytes, a), dev_buf(b.nbytes, b), dev_buf(256 * 256 * 4)
+            args = struct.pack("PPPIIII", lib.wkf_buffer_ptr(ba), lib.wkf_buffer_ptr(bb), lib.wkf_buffer_ptr(bc), 4096, 4096, 4096, 0)
+            grid, block = (c_uint32 * 3)(256, 1, 1), (c_uint32 * 3)(256, 1, 1)
+            us = _raw_timed(lib, dev, lambda: lib.wkf_launch(dev._h, k32, grid, block, 0, args, len(args), None), max(5, launches // 5), 10)
+            rows32.append({"data": label, "us": round(us, 2), "TFLOP/s": round(2 * 4096 ** 3 / us * 1e-6, 1),
+                           "frac_of_f32_peak": round(2 * 4096 ** 3 / us * 1e-6 / F32_MFMA_PEAK_TFLOPS, 4)})
+            for bf in (ba, bb, bc):
+                lib.wkf_buffer_release(bf)
+        out["mfma_only_f32_4096x4096x4096_equivalent"] = rows32
     elif which == "stream":
         n = 1 << 30
         src_b, dst_b, src2_b = dev_buf(n), dev_buf(n), dev_buf(n)
