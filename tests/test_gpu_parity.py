@@ -833,8 +833,8 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 # starts its walk over K at a different tile and wraps around; K with a partial last tile, B^T, edge columns
                 ((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False)]
 # many full tiles over K = 64 or 128: one workgroup per compute unit walks the tiles of the whole batch
-BATCH_SHAPES += [((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True)]
-WHOLE_K = {((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True)}
+BATCH_SHAPES += [((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)]
+WHOLE_K = {((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)}
 ROTATED = {((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False),
            ((8,), 512, 128, 512, False)}
 
