@@ -444,6 +444,7 @@ def test_mat_mul_kernel_choice(wkf, planner):
     # ... and a partly filled last round of it runs in half tiles like that of a full shape (16 x 17 tiles)
     assert detail(4000, 4104, 72, np.float16).endswith("mfma 256x256 tiles edge, last round: 16 tiles as 32 halves of 128 rows")
     assert detail(300, 260, 68, np.float32).endswith("mfma 256x256 tiles edge")
+    assert detail(4096, 4352, 64, np.float32).endswith("mfma 256x256 tiles, last round: 16 tiles as 32 halves of 128 rows")
     # f16 products whose large tiles would fill at most half of the chip take 128 x 128 tiles, two workgroups per compute unit
     assert detail(512, 256, 128, np.float16).endswith("mfma 128x128 tiles")
     assert detail(300, 264, 72, np.float16).endswith("mfma 128x128 tiles")

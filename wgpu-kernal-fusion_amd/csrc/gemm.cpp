@@ -32,6 +32,9 @@ const char* const kGemmF16T128 =
 const char* const kGemmF16Tail =
 #include "kernels/gemm_f16_tail.hip.inc"
     ;
+const char* const kGemmF32Tail =
+#include "kernels/gemm_f32_tail.hip.inc"
+    ;
 const char* const kGemmF16ShortK =
 #include "kernels/gemm_f16_shortk.hip.inc"
     ;
@@ -364,13 +367,14 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     }
   }
   const bool split = slices > 1;
-  // Full f16 tiles that do not fill a whole number of rounds on the chip (the [2048 x 4096] x [4096 x 11008] MLP
+  // Full tiles (f16 also ragged ones) that do not fill a whole number of rounds on the chip (the [2048 x 4096] x [4096 x 11008] MLP
   // product: 344 tiles on 256 compute units): the tiles of the last, partly filled round are computed as two halves
   // of 128 rows each by twice as many workgroups, so that round fills twice as many compute units and takes about
-  // half as long (kernels/gemm_f16_tail.hip.inc).
+  // half as long (kernels/gemm_f16_tail.hip.inc, kernels/gemm_f32_tail.hip.inc).
   size_t ntail = 0, nmain = 0;
   const bool tail_ragged = kind == GemmKind::MfmaF16Edge && K <= (size_t(1) << 21) && N <= (size_t(1) << 22) && N % 8 == 0;
-  if ((kind == GemmKind::MfmaF16 || tail_ragged) && !bt && !t128 && !split && batch == 1 && st_.fusion == FusionMode::Tree && st_.gemm_tail) {
+  if ((kind == GemmKind::MfmaF16 || kind == GemmKind::MfmaF32 || tail_ragged) && !bt && !t128 && !split && batch == 1 &&
+      st_.fusion == FusionMode::Tree && st_.gemm_tail) {
     nmain = tiles / cus * cus;
     ntail = tiles - nmain;
     if (nmain == 0 || ntail * 2 > cus) ntail = 0;
@@ -398,6 +402,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (shortk) sig += K == 64 ? "|whole K in LDS|nt1" : "|whole K in LDS|nt2";
   if (tail) sig += "|last round in half tiles";  // (a ragged shape keeps "|edge" in front of it)
   wkf_kernel* k = kernel(sig, [&] {
+    if (tail && kind == GemmKind::MfmaF32) return std::string(kGemmF32Tail);
     if (tail) return std::string(tail_ragged ? "#define WKF_EDGEBUF 1\n" : "") + kGemmF16Tail;
     std::string src = bt ? "#define WKF_BT 1\n" : "";
     if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (rotk ? "#define WKF_ROTK 1\n" : "") + kGemmF16T128;
