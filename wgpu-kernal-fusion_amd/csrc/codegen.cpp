@@ -195,6 +195,11 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
           o << "(_Float16)__builtin_amdgcn_exp2f((float)" << a << " * 0x1.715476p+0f)";
           break;
         }
+        if (h && exact && policy != MathPolicy::Exact && (in.op == Op::Sin || in.op == Op::Cos)) {
+          // an interior sin / cos on f16: f64 reduction, f32 core, and the f64 core where that cannot decide
+          o << (in.op == Op::Sin ? "wkf_sin_h" : "wkf_cos_h") << "((float)" << a << ")";
+          break;
+        }
         if (h && exact && policy != MathPolicy::Exact && in.op != Op::Sqrt) {
           // an interior transcendental on f16: the f32 library, and the library's f64 routine where that cannot decide
           const std::string f = lib_fn(in.op);
