@@ -73,6 +73,16 @@ int wkf_device_get_fusion(wkf_device* dev);
  * exact != 0: every transcendental op is evaluated in f64 and rounded once. */
 int wkf_device_set_exact_math(wkf_device* dev, int exact);
 
+/* Rows longer than one workgroup's registers (no reference counterpart: the reference's reduce takes a row of any
+ * length in one workgroup, src/reduce.rs:340-350, and its composites read such a row once per stage).  Here a row
+ * that fits the registers of up to 256 workgroups is computed in ONE launch that reads it once: the workgroups of
+ * a row exchange their folded values through memory and wait for each other (all of them are resident: the grid
+ * never exceeds four workgroups per compute unit).  The wait is bounded: a lane polls at most `spin_polls` times
+ * over the whole kernel (0 = the default, 2^20; the top bit is a test hook that keeps one workgroup per row
+ * silent) and then gives up; the next wkf_tensor_as_slice on the device then fails with WKF_ERR_HIP instead of
+ * handing out a result.  enabled = 0 goes back to one launch per stage (or one workgroup streaming each row). */
+int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls);
+
 /* Per-kernel GPU timestamps (PerformanceQueries, src/query.rs:50-126: the reference
  * attaches one to every kernel).  On by default; a caller that only wants results can
  * switch the hipEvent pair per launch off. */

@@ -567,15 +567,37 @@ def test_row_kernels_on_rows_that_do_not_split_evenly(gpu, rows, n, dtype):
     assert np.allclose(got[2].astype(np.float64), total, rtol=1e-5 if dtype == np.float32 else 4e-3)
 
 
+class row_teams:
+    """Row kernels that spread a long row over the registers of several blocks: on (the default) or off for a while."""
+
+    def __init__(self, gpu, on, spin_polls=0):
+        self.gpu, self.on, self.spin = gpu, on, spin_polls
+
+    def __enter__(self):
+        self.gpu.set_row_teams(self.on, self.spin)
+
+    def __exit__(self, *exc):
+        self.gpu.set_row_teams(True, 0)
+        return False
+
+
 LONG_ROWS = [(256, 100003, np.float32), (258, 131076, np.float32), (257, 70000, np.float32), (256, 140002, np.float16),
              (261, 131080, np.float16)]
 
 
+@pytest.mark.parametrize("teams", [True, False], ids=["teams", "streamed"])
 @pytest.mark.parametrize("rows,n,dtype", LONG_ROWS, ids=[f"{r}x{n}_{np.dtype(d).name}" for r, n, d in LONG_ROWS])
-def test_rows_longer_than_a_blocks_registers_stay_one_kernel(gpu, rows, n, dtype):
-    # Rows beyond 65536 floats do not fit the registers of a block: with enough rows to occupy the chip one block
-    # per row streams its row once per stage and once more for the result, in ONE launch (the reference's reduce
-    # takes any length in one kernel, src/reduce.rs:340-350); odd lengths take narrower vectors.
+def test_rows_longer_than_a_blocks_registers_stay_one_kernel(gpu, rows, n, dtype, teams):
+    # Rows beyond 65536 floats do not fit the registers of a block.  They are spread over the registers of a team
+    # of blocks that exchange their folds (ONE launch, the row read once); without teams, and with enough rows to
+    # occupy the chip, one block per row streams its row once per stage and once more for the result, also in one
+    # launch (the reference's reduce takes any length in one kernel, src/reduce.rs:340-350); odd lengths take
+    # narrower vectors.
+    with row_teams(gpu, teams):
+        _long_rows_one_kernel(gpu, rows, n, dtype, "teams of" if teams else "streamed")
+
+
+def _long_rows_one_kernel(gpu, rows, n, dtype, mark):
     x = data((rows, n), -3, 3, dtype, rows * 11 + n)
     w = data((n,), 0.5, 1.5, dtype, n + 1)
     api = HipAPI(gpu)
@@ -588,7 +610,7 @@ def test_rows_longer_than_a_blocks_registers_stay_one_kernel(gpu, rows, n, dtype
         want.append(ox.layer_norm(ow, 1e-5).to_numpy())
     got = hip_values_many(progs)
     for p in progs:
-        assert [k.kind for k in p.kernels()] == ["row"] and "streamed" in p.kernels()[0].detail, [k.detail for k in p.kernels()]
+        assert [k.kind for k in p.kernels()] == ["row"] and mark in p.kernels()[0].detail, [k.detail for k in p.kernels()]
     rtol = 1e-5 if dtype == np.float32 else 2e-3
     for i in range(len(got)):
         assert got[i].shape == want[i].shape
@@ -606,11 +628,18 @@ def test_rows_longer_than_a_blocks_registers_stay_one_kernel(gpu, rows, n, dtype
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float16])
 @pytest.mark.parametrize("rows,n", [(5, 100003), (64, 65540), (1, 1 << 20), (100, 70000), (127, 65600), (3, 70001)])
-def test_few_long_rows_are_split_into_parts(gpu, rows, n, dtype):
+@pytest.mark.parametrize("teams", [True, False], ids=["teams", "split"])
+def test_few_long_rows_are_split_into_parts(gpu, rows, n, dtype, teams):
     # with only a few rows a block per row would leave most compute units idle: every row is cut into parts with a
-    # block each and every stage becomes one launch that leaves its parts' values to the next (softmax: the online
-    # pair of max and sum, then the result = two launches; layer_norm: three).  The reference's reduce takes any
-    # length in one kernel (src/reduce.rs:340-350).
+    # block each.  In a team the parts stay in the blocks' registers and the blocks exchange their folds (one
+    # launch); without teams every stage becomes one launch that leaves its parts' values to the next (softmax: the
+    # online pair of max and sum, then the result = two launches; layer_norm: three).  The reference's reduce takes
+    # any length in one kernel (src/reduce.rs:340-350).
+    with row_teams(gpu, teams):
+        _few_long_rows(gpu, rows, n, dtype, teams)
+
+
+def _few_long_rows(gpu, rows, n, dtype, teams):
     if dtype == np.float16:
         # as many bytes as the f32 case, so that the rows are too long for a block's registers, but no more
         # than about 390 000 elements: beyond that sum(exp(x - max)) of these inputs overflows f16
@@ -628,10 +657,12 @@ def test_few_long_rows_are_split_into_parts(gpu, rows, n, dtype):
         want.append(ox.layer_norm(ow, 1e-5).to_numpy())
         launches.append(2)
     got = hip_values_many(progs)
-    for p, count in zip(progs, launches):
+    for i, (p, count) in enumerate(zip(progs, launches)):
         ks = p.kernels()
-        assert [k.kind for k in ks] == ["row"] * count, [(k.kind, k.detail) for k in ks]
-        assert all("rows split in" in k.detail for k in ks), [k.detail for k in ks]
+        # (layer_norm holds two operands per lane, so its teams are twice as large: beyond 256 parts it stays split)
+        team = teams and (i == 0 or "teams of" in ks[0].detail)
+        assert [k.kind for k in ks] == ["row"] * (1 if team else count), [(k.kind, k.detail) for k in ks]
+        assert all(("teams of" if team else "rows split in") in k.detail for k in ks), [k.detail for k in ks]
     rtol = 1e-5 if dtype == np.float32 else 2e-3
     for i in range(len(got)):
         assert got[i].shape == want[i].shape
@@ -640,7 +671,29 @@ def test_few_long_rows_are_split_into_parts(gpu, rows, n, dtype):
     assert np.array_equal(np.argmax(got[0], 1), np.argmax(x, 1))
 
 
-def test_split_rows_of_a_view_and_with_stages_that_do_not_pair(gpu):
+@pytest.mark.parametrize("teams", [True, False], ids=["teams", "split"])
+def test_split_rows_of_a_view_and_with_stages_that_do_not_pair(gpu, teams):
+    with row_teams(gpu, teams):
+        _rows_of_a_view_and_stages_that_do_not_pair(gpu, teams)
+
+
+def test_a_team_that_gives_up_waiting_is_reported_at_read_back(gpu):
+    # The blocks of a team wait for each other's values a bounded number of polls.  Here part 0 of every row stays
+    # silent (the top bit of the bound) and the bound is tiny, so the lanes that wait for it give up, every block
+    # still runs to its end, and the read-back refuses the result; the next computation is clean again.
+    x = data((4, 100000), -3, 3, np.float32, 21)
+    api = HipAPI(gpu)
+    with row_teams(gpu, True, (1 << 31) | 64):
+        t = api.tensor(x).softmax_last_dim()
+        with pytest.raises(Exception, match="gave up waiting"):
+            hip_values(t)
+    t = api.tensor(x).softmax_last_dim()
+    got = hip_values(t)
+    assert "teams of" in t.kernels()[0].detail
+    assert np.allclose(got, OTensor(x).softmax_last_dim().to_numpy(), rtol=1e-5, atol=1e-9)
+
+
+def _rows_of_a_view_and_stages_that_do_not_pair(gpu, teams):
     # the operand is a column block of a wider matrix (row stride != row length)
     big = data((6, 3 * 100000), -2, 2, np.float32, 5)
     api = HipAPI(gpu)
@@ -648,7 +701,8 @@ def test_split_rows_of_a_view_and_with_stages_that_do_not_pair(gpu):
     t = api.tensor(big).slice([(0, 6), (100000, 200000)]).layer_norm(api.tensor(w), 1e-5)
     got = hip_values(t)
     want = OTensor(big).slice([(0, 6), (100000, 200000)]).layer_norm(OTensor(w), 1e-5).to_numpy()
-    assert len(t.kernels()) == 2 and all("rows split in" in k.detail for k in t.kernels()), [k.detail for k in t.kernels()]
+    mark = "teams of" if teams else "rows split in"
+    assert len(t.kernels()) == (1 if teams else 2) and all(mark in k.detail for k in t.kernels()), [k.detail for k in t.kernels()]
     assert np.allclose(got, want, rtol=1e-5, atol=1e-7)
     # softmax of 2x: the maximum is not of the operand itself, so max and sum stay passes of their own (three launches)
     x = data((9, 90000), -3, 3, np.float32, 8)
@@ -656,7 +710,8 @@ def test_split_rows_of_a_view_and_with_stages_that_do_not_pair(gpu):
     got = hip_values(t)
     want = (OTensor(x) * 0.5).softmax_last_dim().to_numpy()
     ks = t.kernels()
-    assert len(ks) == 3 and all("rows split in" in k.detail and "in one pass" not in k.detail for k in ks), [k.detail for k in ks]
+    assert len(ks) == (1 if teams else 3), [k.detail for k in ks]
+    assert all(mark in k.detail and "in one pass" not in k.detail and "in one exchange" not in k.detail for k in ks), [k.detail for k in ks]
     assert np.allclose(got, want, rtol=1e-5, atol=1e-9)
 
 

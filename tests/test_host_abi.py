@@ -408,17 +408,39 @@ def test_row_kernel_takes_rows_that_do_not_split_evenly(wkf, planner):
     assert "vec=8" in detail((8, 2880), np.float16, sm) and "vec=4" in detail((8, 11004), np.float16, sm)
     # rows of a view that start off the vector grid take narrower vectors instead of three kernels
     assert "vec=1" in detail((8, 4096), np.float32, lambda t: t.slice([(0, 8), (1, 4095)]).softmax_last_dim())
-    # beyond what 1024 lanes hold in registers a few rows are split into parts: one launch for the online pair of
-    # max and sum over every part, one that folds a row's parts and writes the result
-    long_rows = _x(wkf, planner, (2, 65537), np.float32).softmax_last_dim()
-    assert _kinds(long_rows) == ["row", "row"]
-    details = [k.detail for k in long_rows.kernels()]
-    assert details[0].endswith("streamed (max and sum in one pass), rows split in 65 parts of 1024 vectors: launch 1 of 2"), details
-    assert details[1].endswith("launch 2 of 2") and long_rows.kernels()[0].signature.endswith("|split0")
-    assert long_rows.kernels()[1].signature.endswith("|split2")
-    # 256 rows or more stream with a block per row, in one launch
-    many = _x(wkf, planner, (256, 65537), np.float32).softmax_last_dim()
-    assert _kinds(many) == ["row"] and many.kernels()[0].detail.endswith("streamed (max and sum in one pass)")
+    # beyond what 1024 lanes hold in registers a row is spread over the registers of a team of blocks that exchange
+    # their folds: one launch, the row read once; the grid never exceeds four blocks per compute unit (1024 here)
+    assert detail((2, 65537), np.float32, sm).endswith(
+        "vectors_per_lane=8 stages=2 operands=2, max and sum in one exchange, rows in the registers of teams of 33 blocks, 2 teams")
+    assert detail((256, 65537), np.float32, sm).endswith("rows in the registers of teams of 33 blocks, 31 teams")
+    assert detail((64, 262144), np.float32, sm).endswith("rows in the registers of teams of 32 blocks, 32 teams")
+    team = _x(wkf, planner, (3, 200000), np.float16).softmax_last_dim()
+    assert _kinds(team) == ["row"] and team.kernels()[0].signature.endswith("|online|team") and team.kernels()[0].detail.endswith("teams of 13 blocks, 3 teams")
+    # two operands: half the vectors per lane each; a stage that does not pair with the next: one exchange per stage
+    two = _x(wkf, planner, (4, 80000), np.float32)
+    two = (two + _x(wkf, planner, (4, 80000), np.float32, seed=1)).softmax_last_dim()
+    assert _kinds(two) == ["row"] and "vectors_per_lane=4" in two.kernels()[0].detail and "teams of 20 blocks" in two.kernels()[0].detail
+    norm = _x(wkf, planner, (4, 80000), np.float32).layer_norm(_x(wkf, planner, (80000,), np.float32, seed=2), 1e-5)
+    assert _kinds(norm) == ["row"], [k.detail for k in norm.kernels()]
+    assert "in one exchange" not in norm.kernels()[0].detail and "teams of" in norm.kernels()[0].detail
+    # rows of more than 256 parts (2 M floats) and devices with teams switched off keep the kernels below
+    planner.set_row_teams(False)
+    try:
+        # a few rows are split into parts: one launch for the online pair of max and sum over every part, one that
+        # folds a row's parts and writes the result
+        long_rows = _x(wkf, planner, (2, 65537), np.float32).softmax_last_dim()
+        assert _kinds(long_rows) == ["row", "row"]
+        details = [k.detail for k in long_rows.kernels()]
+        assert details[0].endswith("streamed (max and sum in one pass), rows split in 65 parts of 1024 vectors: launch 1 of 2"), details
+        assert details[1].endswith("launch 2 of 2") and long_rows.kernels()[0].signature.endswith("|split0")
+        assert long_rows.kernels()[1].signature.endswith("|split2")
+        # 256 rows or more stream with a block per row, in one launch
+        many = _x(wkf, planner, (256, 65537), np.float32).softmax_last_dim()
+        assert _kinds(many) == ["row"] and many.kernels()[0].detail.endswith("streamed (max and sum in one pass)")
+    finally:
+        planner.set_row_teams(True)
+    wide = _x(wkf, planner, (2, (1 << 21) + 4096), np.float32).softmax_last_dim()
+    assert _kinds(wide) == ["row", "row"] and "rows split in" in wide.kernels()[0].detail
     # rows that are short but too many vectors for the lanes' registers (fewer than 1024 vectors never are) stay decomposed
     assert _kinds(_x(wkf, planner, (2, 70000), np.float32).max(1)) == ["red_row", "red_row"]
 

@@ -957,6 +957,7 @@ std::string row_signature(const RowSpec& s) {
   if (s.streamed) o << "|streamed";
   if (s.online_max_sum) o << "|online";
   if (s.split) o << "|split" << s.split_phase;
+  if (s.team) o << "|team";
   return o.str();
 }
 
@@ -991,7 +992,8 @@ std::string row_source(const RowSpec& s) {
     if (round_h) o << kRoundH;
   }
   o << kRowHelpers;
-  o << "struct Args { void* p[" << K + NOUT + (s.split ? 1 : 0) << "]; u32 nrows; " << (s.ragged || s.streamed ? "u32 nvec; " : "") << (s.split ? "u32 parts; u32 chunk; " : "")
+  o << "struct Args { void* p[" << K + NOUT + (s.split ? 1 : 0) + (s.team ? 2 : 0) << "]; u32 nrows; " << (s.ragged || s.streamed || s.team ? "u32 nvec; " : "")
+    << (s.split ? "u32 parts; u32 chunk; " : "") << (s.team ? "u32 parts; u32 spin; " : "")
     << "u32 oshape[" << std::max(1, Ro) << "]; u32 off[" << K + NOUT
     << "]; u32 ostride[" << K + NOUT << "][" << std::max(1, Ro) << "]; float c[" << std::max(1, nc) << "]; };\n";
   // operand types as every program sees them: the K full operands, then one scalar per earlier stage
@@ -1005,6 +1007,232 @@ std::string row_source(const RowSpec& s) {
   }
   if (!s.store_scalars) emit_program(o, s.final, "wkf_final", types, store_policy);
 
+  if (s.team) {
+    // ---- rows longer than the registers of a block, held in the registers of a TEAM of blocks ----
+    // Block b works on part b % parts of rows b / parts, b / parts + teams, ...: its share of the row (NV vectors
+    // per lane and operand) comes into registers once and stays there.  Every stage is folded inside the block,
+    // lane 192 puts the block's value into slot [stage][row][part] (64 bits: the value and a "written" mark, one
+    // atomic store), the lanes of wave 3 read the slots of all parts, waiting until each is written, fold them and
+    // hand the row's value to the other waves through the LDS.  The NEXT row's loads are issued before this row
+    // is folded and travel meanwhile (memory operations of a wave return in order, so wave 3 sees a slot only
+    // after its own share of those loads has landed; a wave that held no data would see it sooner, but a quarter
+    // fewer registers per round cost more than that wait: 155 us against 117 for softmax over [256, 262144]).
+    // All blocks of a team are resident together: blocks start in the order of their index, a team's blocks are
+    // neighbours, and the host sizes the grid for four blocks per compute unit, which the launch bounds
+    // guarantee; even a chip that held fewer would hold whole teams first, and those run to their end without
+    // anyone else.  So the wait ends; it is bounded all the same (a.spin polls per lane over the whole kernel),
+    // and a lane that gives up counts itself in *gave_up, which the host reads before it hands any result out.
+    // A slot is written once and never reused.  Softmax's max / sum pair crosses in one exchange: the sums
+    // travel relative to their part's maximum and are rescaled to the row's.  (Starting every other team half a
+    // row late, so that one half moves data while the other waits, only added the delay: 117 -> 122-126 us.)
+    const int TD = 256;  // data lanes
+    const int XL = 192;  // first lane of the wave that also talks to the other blocks
+    const int NW = TD / 64;
+    if (T != TD || B != 256 || s.store_scalars || S < 1) throw Error(WKF_ERR_INVALID_ARG, "row_source: team kernels are blocks of 256 lanes with a result row");
+    o << "typedef unsigned long long u64;\n";
+    o << "static __device__ __forceinline__ void wkf_team_put(u64* slot, float v) {\n"
+         "  __hip_atomic_store(slot, 0x100000000ull | (u64)__builtin_bit_cast(u32, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n}\n";
+    // up to two slots a poll (they travel together); `n` = 1 or 2
+    o << "static __device__ __forceinline__ void wkf_team_get(u64* slot_a, u64* slot_b, float& va, float& vb, u32& polls_left, u64* gave_up) {\n"
+         "  for (;;) {\n"
+         "    const u64 wa = __hip_atomic_load(slot_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n"
+         "    const u64 wb = __hip_atomic_load(slot_b, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n"
+         "    va = __builtin_bit_cast(float, (u32)wa);\n"
+         "    vb = __builtin_bit_cast(float, (u32)wb);\n"
+         "    if ((wa >> 32) != 0ull && (wb >> 32) != 0ull) return;\n"
+         "    if (polls_left == 0u) {\n"
+         "      __hip_atomic_fetch_add(gave_up, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n"
+         "      return;\n"
+         "    }\n"
+         "    polls_left--;\n"
+         "    __builtin_amdgcn_s_sleep(2);\n"
+         "  }\n}\n";
+    // every sync point of a row has LDS words of its own: a word is written again only one row later, with at
+    // least one barrier between any wave's read of it and that write
+    int nsync = 0;
+    for (int k = 0; k < S; k++) nsync += 2;
+    o << "extern \"C\" __global__ void __launch_bounds__(256, 4) WKF_ENTRY(const Args a) {\n";
+    o << "  __shared__ float wkf_lds[" << nsync << "][4];\n";
+    o << "  const u32 t = threadIdx.x;\n";
+    o << "  const bool data_wave = __builtin_amdgcn_readfirstlane(threadIdx.x) < " << TD << "u;  // uniform over the wave\n";
+    o << "  const bool talk_wave = __builtin_amdgcn_readfirstlane(threadIdx.x) >= " << XL << "u;\n";
+    o << "  const u32 part = blockIdx.x % a.parts;\n";
+    o << "  const u32 teams = gridDim.x / a.parts;\n";
+    o << "  u64* const slots = (u64*)a.p[" << K + 1 << "];\n";
+    o << "  u64* const gave_up = (u64*)a.p[" << K + 2 << "];\n";
+    o << "  u32 polls_left = a.spin & 0x7fffffffu;\n";
+    o << "  const bool mute = (a.spin >> 31) != 0u && part == 0u;  // host-side test of the give-up path: part 0 never writes its slots\n";
+    for (int k = 0; k < S; k++) {
+      const bool online = s.online_max_sum && k < 2;
+      o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(online ? (k == 0 ? ReduceOp::Max : ReduceOp::Sum) : s.stages[k].rop)
+        << "; };\n";
+    }
+    auto stage_rop = [&](int k) { return s.online_max_sum && k < 2 ? (k == 0 ? ReduceOp::Max : ReduceOp::Sum) : s.stages[k].rop; };
+    // the element offset of operand k's row `row`, through index variables with the suffix `sfx`
+    auto emit_indices = [&](const char* ind, const char* row, const char* sfx) {
+      if (Ro > 0) {
+        o << ind << "u32 rem" << sfx << " = " << row << ";\n";
+        for (int d = Ro - 1; d > 0; d--)
+          o << ind << "const u32 i" << d << sfx << " = rem" << sfx << " % a.oshape[" << d << "]; rem" << sfx << " /= a.oshape[" << d << "];\n";
+        o << ind << "const u32 i0" << sfx << " = rem" << sfx << ";\n";
+      }
+    };
+    auto base_expr = [&](int k, const char* sfx) {
+      std::ostringstream e;
+      e << "a.off[" << k << "]";
+      for (int d = 0; d < Ro; d++) e << " + i" << d << sfx << " * a.ostride[" << k << "][" << d << "]";
+      return e.str();
+    };
+    // The loads of one row into the variables <x|s><dst>k_j.  They are buffer loads without a branch around them, so
+    // that the compiler can count the loads in flight and wait for exactly those it needs (after a load under
+    // `if` it waits for all of them): the resource ends where the row ends, or has no extent at all when there is
+    // no such row or the wave holds no data (`has`), and a load past its end returns zeros without touching memory.
+    auto buffer_load = [&](DType dt, int lanes, const std::string& rsrc, const std::string& off) {
+      const size_t bytes = dtype_size(dt) * size_t(lanes);
+      const char* fn = bytes == 16 ? "b128" : bytes == 8 ? "b64" : bytes == 4 ? "b32" : "b16";
+      return "__builtin_bit_cast(" + vtype(dt, lanes) + ", __builtin_amdgcn_raw_buffer_load_" + fn + "(" + rsrc + ", " + off + ", 0, 2))";
+    };
+    auto emit_loads = [&](const char* ind, const char* row, const char* sfx, const char* dst, const char* has) {
+      emit_indices(ind, row, sfx);
+      for (int k = 0; k < K; k++) {
+        const char* ct = ctype(s.in[k].dtype);
+        const size_t es = dtype_size(s.in[k].dtype);
+        const bool scalar = s.in[k].axis_stride == 0;
+        o << ind << "const __amdgpu_buffer_rsrc_t rs" << k << sfx << " = __builtin_amdgcn_make_buffer_rsrc((void*)(((const " << ct << "*)a.p[" << k
+          << "]) + (" << base_expr(k, sfx) << ")), 0, " << has << " ? " << (scalar ? std::to_string(es) + "u" : "a.nvec * " + std::to_string(es * size_t(V)) + "u")
+          << " : 0u, 0x00020000);\n";
+        if (scalar) {
+          o << ind << "s" << dst << k << " = " << buffer_load(s.in[k].dtype, 1, "rs" + std::to_string(k) + sfx, "0u") << ";\n";
+        } else {
+          for (int j = 0; j < NV; j++)
+            o << ind << "x" << dst << k << "_" << j << " = "
+              << buffer_load(s.in[k].dtype, V, "rs" + std::to_string(k) + sfx, "j" + std::to_string(j) + " * " + std::to_string(es * size_t(V)) + "u") << ";\n";
+        }
+      }
+    };
+    auto declare = [&](const char* ind, const char* dst) {
+      for (int k = 0; k < K; k++) {
+        if (s.in[k].axis_stride == 0) o << ind << ctype(s.in[k].dtype) << " s" << dst << k << ";\n";
+        else
+          for (int j = 0; j < NV; j++) o << ind << vtype(s.in[k].dtype, V) << " x" << dst << k << "_" << j << ";\n";
+      }
+    };
+    for (int j = 0; j < NV; j++)
+      o << "  const u32 j" << j << " = (part * " << NV << "u + " << j << "u) * " << TD << "u + t; const bool ok" << j << " = data_wave && j" << j << " < a.nvec;\n";
+    o << "  const u32 row0 = blockIdx.x / a.parts;\n";
+    declare("  ", "");
+    o << "  {\n";
+    emit_loads("    ", "min(row0, a.nrows - 1u)", "f", "", "(data_wave && row0 < a.nrows)");
+    o << "  }\n";
+    o << "  for (u32 row = row0; row < a.nrows; row += teams) {\n";
+    declare("  ", "n");
+    o << "  {\n";
+    emit_loads("    ", "min(row + teams, a.nrows - 1u)", "n", "n", "(data_wave && row + teams < a.nrows)");
+    o << "  }\n";
+    emit_indices("  ", "row", "");
+    auto call_args = [&](int j, int e, int nscalars) {
+      std::ostringstream c;
+      for (int k = 0; k < K; k++) {
+        if (s.in[k].axis_stride == 0) c << "s" << k;
+        else {
+          c << "x" << k << "_" << j;
+          if (V > 1) c << "[" << e << "]";
+        }
+        c << ", ";
+      }
+      for (int q = 0; q < nscalars; q++) c << "r" << q << ", ";
+      return c.str();
+    };
+    int sync = 0;
+    // acc<k> over this lane's vectors, then over the block's data waves; every wave gets the value
+    auto own_fold = [&](int k, const char* ind) {
+      // (no branch: a vector past the end of the row came back as zeros and folds as the seed)
+      const char* seed = seed_text(stage_rop(k));
+      for (int j = 0; j < NV; j++)
+        for (int e = 0; e < V; e++)
+          o << ind << "acc" << k << " = fold" << k << "(ok" << j << " ? (float)wkf_pre" << k << "(" << call_args(j, e, k) << "a.c + " << pre_off[k] << ") : "
+            << seed << ", acc" << k << ");\n";
+      o << ind << "acc" << k << " = wkf_lanes_fold_with<64>(acc" << k << ", fold" << k << ");\n";
+      o << ind << "if (data_wave && (t & 63u) == 0u) wkf_lds[" << sync << "][t >> 6] = acc" << k << ";\n";
+      o << ind << "__syncthreads();\n";
+      o << ind << "acc" << k << " = fold" << k << "(wkf_lds[" << sync << "][0], fold" << k << "(wkf_lds[" << sync << "][1], wkf_lds[" << sync << "][2]));\n";
+      if (NW == 4) o << ind << "acc" << k << " = fold" << k << "(wkf_lds[" << sync << "][3], acc" << k << ");\n";
+      sync++;
+    };
+    auto slot = [&](int k, const char* who) { return "slots + ((" + std::to_string(k) + "u * a.nrows + row) * a.parts + " + who + ")"; };
+    auto post = [&](int k) {
+      o << "  const " << ctype(s.stages[k].post.result_dtype()) << " r" << k << " = wkf_post" << k << "((" << ctype(s.stages[k].pre.result_dtype())
+        << ")acc" << k << ", a.c + " << post_off[k] << ");\n";
+    };
+    for (int k = 0; k < S; k++) {
+      if (s.online_max_sum && k == 0) {
+        o << "  float acc0 = " << seed_text(ReduceOp::Max) << ", acc1 = " << seed_text(ReduceOp::Sum) << ";\n";
+        own_fold(0, "  ");
+        o << "  {\n    const " << ctype(s.stages[0].post.result_dtype()) << " r0 = wkf_post0((" << ctype(s.stages[0].pre.result_dtype())
+          << ")acc0, a.c + " << post_off[0] << ");  // this part's maximum\n";
+        own_fold(1, "    ");
+        o << "  }\n";
+        o << "  if (talk_wave) {\n";
+        o << "    if (t == " << XL << "u && !mute) {\n      wkf_team_put(" << slot(0, "part") << ", acc0);\n      wkf_team_put(" << slot(1, "part") << ", acc1);\n    }\n";
+        o << "    float row_max = " << seed_text(ReduceOp::Max) << ", row_sum = 0.0f;\n";
+        o << "    for (u32 p = t - " << XL << "u; p < a.parts; p += 64u) {\n";
+        o << "      float part_max, part_sum;\n";
+        o << "      wkf_team_get(" << slot(0, "p") << ", " << slot(1, "p") << ", part_max, part_sum, polls_left, gave_up);\n";
+        o << "      const float m = fmaxf(part_max, row_max);\n";
+        o << "      row_sum = row_sum * expf(row_max - m) + part_sum * expf(part_max - m);\n";
+        o << "      row_max = m;\n";
+        o << "    }\n";
+        o << "    const float lane_max = row_max;\n";
+        o << "    row_max = wkf_lanes_fold_with<64>(row_max, fold0);\n";
+        o << "    row_sum = wkf_lanes_fold_with<64>(row_sum * expf(lane_max - row_max), fold1);\n";
+        o << "    if (t == " << XL << "u) {\n      wkf_lds[" << sync << "][0] = row_max;\n      wkf_lds[" << sync << "][1] = row_sum;\n    }\n";
+        o << "  }\n";
+        o << "  __syncthreads();\n";
+        o << "  acc0 = wkf_lds[" << sync << "][0];\n  acc1 = wkf_lds[" << sync << "][1];\n";
+        sync++;
+        post(0);
+        post(1);
+        k = 1;
+        continue;
+      }
+      o << "  float acc" << k << " = " << seed_text(s.stages[k].rop) << ";\n";
+      own_fold(k, "  ");
+      o << "  if (talk_wave) {\n";
+      o << "    if (t == " << XL << "u && !mute) wkf_team_put(" << slot(k, "part") << ", acc" << k << ");\n";
+      o << "    float v = " << seed_text(s.stages[k].rop) << ";\n";
+      o << "    for (u32 p = t - " << XL << "u; p < a.parts; p += 64u) {\n";
+      o << "      float pa, pb;\n";
+      o << "      wkf_team_get(" << slot(k, "p") << ", " << slot(k, "p") << ", pa, pb, polls_left, gave_up);\n";
+      o << "      v = fold" << k << "(pa, v);\n";
+      o << "    }\n";
+      o << "    v = wkf_lanes_fold_with<64>(v, fold" << k << ");\n";
+      o << "    if (t == " << XL << "u) wkf_lds[" << sync << "][0] = v;\n";
+      o << "  }\n";
+      o << "  __syncthreads();\n";
+      o << "  acc" << k << " = wkf_lds[" << sync << "][0];\n";
+      sync++;
+      post(k);
+    }
+    const char* ot = ctype(s.out_dtype);
+    std::string ovt = vtype(s.out_dtype, V);
+    o << "  " << ot << "* qo = ((" << ot << "*)a.p[" << K << "]) + (" << base_expr(K, "") << ");\n";
+    for (int j = 0; j < NV; j++) {
+      o << "  if (ok" << j << ") {\n    " << ovt << " ov;\n";
+      for (int e = 0; e < V; e++) {
+        o << "    ov";
+        if (V > 1) o << "[" << e << "]";
+        o << " = wkf_final(" << call_args(j, e, S) << "a.c + " << final_off << ");\n";
+      }
+      o << "    __builtin_nontemporal_store(ov, (" << ovt << "*)(qo + j" << j << " * " << V << "u));\n  }\n";
+    }
+    for (int k = 0; k < K; k++) {
+      if (s.in[k].axis_stride == 0) o << "  s" << k << " = sn" << k << ";\n";
+      else
+        for (int j = 0; j < NV; j++) o << "  x" << k << "_" << j << " = xn" << k << "_" << j << ";\n";
+    }
+    o << "  }\n}\n";
+    return o.str();
+  }
   o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") WKF_ENTRY(const Args a) {\n";
   if (T > 64) o << "  __shared__ float wkf_partial[" << std::max(1, S) << "][" << B / 64 << "];\n";
   o << "  const u32 t = threadIdx.x % " << T << "u;\n";
@@ -1263,15 +1491,19 @@ std::string row_source(const RowSpec& s) {
 std::vector<unsigned char> row_pack_args(const RowSpec& s, const RowArgs& a) {
   const size_t K = s.in.size(), Ro = size_t(s.outer_rank);
   const size_t NP = K + (s.store_scalars ? s.stages.size() : 1);
-  if (a.ptrs.size() != NP + (s.split ? 1 : 0) || a.oshape.size() != Ro || a.offsets.size() != NP || a.ostrides.size() != NP)
+  if (a.ptrs.size() != NP + (s.split ? 1 : 0) + (s.team ? 2 : 0) || a.oshape.size() != Ro || a.offsets.size() != NP || a.ostrides.size() != NP)
     throw Error(WKF_ERR_INVALID_ARG, "row_pack_args: argument arity does not match the kernel");
   std::vector<unsigned char> b;
   for (void* p : a.ptrs) putp(b, p);
   put32(b, a.nrows);
-  if (s.ragged || s.streamed) put32(b, a.nvec);
+  if (s.ragged || s.streamed || s.team) put32(b, a.nvec);
   if (s.split) {
     put32(b, a.parts);
     put32(b, a.chunk);
+  }
+  if (s.team) {
+    put32(b, a.parts);
+    put32(b, a.spin);
   }
   for (size_t d = 0; d < std::max<size_t>(1, Ro); d++) put32(b, d < Ro ? a.oshape[d] : 1);
   for (uint32_t v : a.offsets) put32(b, v);

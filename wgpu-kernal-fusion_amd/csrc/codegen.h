@@ -160,6 +160,13 @@ struct RowSpec {
   // the result.  Each first folds the parts of the stages before it.  An online pair is one kernel (phase 0).
   bool split = false;
   int split_phase = 0;
+  // team (rows with a `final`, 256 lanes): the row is longer than a block's registers hold but fits those of `parts`
+  // blocks (a launch argument) with `vectors_per_lane` vectors per lane each.  One launch, the row is read once:
+  // the blocks of a row exchange their folded values through 64-bit slots [stages][rows][parts] (second to last
+  // pointer argument, zero-filled by the caller) and wait for each other, which needs every block of the grid
+  // resident: the grid is teams * parts blocks with at most four blocks per compute unit, and a team walks rows
+  // team, team + teams, ...  The last pointer argument counts the lanes that gave up waiting (see `spin`).
+  bool team = false;
   std::vector<ReduceOperandSpec> in;    // axis_stride 1 (row in registers) or 0 (one scalar per row)
   std::vector<RowStage> stages;
   Program final;                        // same operand numbering as a stage's pre
@@ -172,10 +179,12 @@ struct RowSpec {
 std::string row_signature(const RowSpec& s);
 std::string row_source(const RowSpec& s);
 struct RowArgs {
-  std::vector<void*> ptrs;                        // inputs..., out (store_scalars: one out per stage)[, the parts of a split row]
+  std::vector<void*> ptrs;                        // inputs..., out (store_scalars: one out per stage)[, the parts of a split row][, slots, give-up count of a team]
   uint32_t nrows;
   uint32_t nvec = 0;                              // ragged and streamed kernels only: vectors per row
-  uint32_t parts = 0, chunk = 0;                  // split kernels only: parts per row, vectors per part
+  uint32_t parts = 0, chunk = 0;                  // split kernels: parts per row, vectors per part; team kernels: parts
+  uint32_t spin = 0;                              // team kernels: polls a lane may spend waiting over the whole kernel (low 31 bits);
+                                                  // top bit: part 0 never writes its slots (test of the give-up path)
   std::vector<uint32_t> oshape;
   std::vector<uint32_t> offsets;                  // per operand incl. outputs
   std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. outputs, per outer dim

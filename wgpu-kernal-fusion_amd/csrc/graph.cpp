@@ -222,7 +222,64 @@ NodeP Resolver::slice_through(const NodeP& n, size_t axis, size_t start, size_t 
 }  // namespace wkf
 // hip_ffi.cpp: the device's static scratch array as a buffer handle (a new reference) and its size
 wkf_buffer* wkf_scratch_(wkf_device* dev, size_t* bytes);
+// hip_ffi.cpp: `fn` is called when a device is about to be destroyed, to drop state (and buffers) kept for it
+void wkf_add_destroy_hook_(void (*fn)(wkf_device*));
+// hip_ffi.cpp: wkf_device_destroy has been called and only live buffers keep the device
+bool wkf_device_closing_(wkf_device* dev);
 namespace wkf {
+
+namespace {
+// One 8-byte word per device for team row kernels (the lanes that gave up waiting), allocated at the first such
+// launch and kept until the device is destroyed; `pending` = a team kernel ran since the word was last read.
+struct TeamWord {
+  BufRef buf;
+  bool pending = false;
+};
+std::mutex g_team_mu;
+std::unordered_map<wkf_device*, TeamWord> g_team;
+void team_forget(wkf_device* dev) {
+  TeamWord w;
+  {
+    std::lock_guard<std::mutex> lock(g_team_mu);
+    auto it = g_team.find(dev);
+    if (it == g_team.end()) return;
+    w = std::move(it->second);
+    g_team.erase(it);
+  }
+}  // the buffer is released here, outside the lock
+void* team_word(wkf_device* dev) {
+  static const bool hooked = (wkf_add_destroy_hook_(&team_forget), true);
+  (void)hooked;
+  std::lock_guard<std::mutex> lock(g_team_mu);
+  TeamWord& w = g_team[dev];
+  if (!w.buf) {
+    wkf_buffer* b = nullptr;
+    check(wkf_buffer_alloc(dev, 8, 1, &b));
+    w.buf = BufRef(b);
+  }
+  w.pending = true;
+  return wkf_buffer_ptr(w.buf.get());
+}
+}  // namespace
+
+void team_check(wkf_device* dev) {
+  BufRef buf;
+  {
+    std::lock_guard<std::mutex> lock(g_team_mu);
+    auto it = g_team.find(dev);
+    if (it == g_team.end() || !it->second.pending) return;
+    it->second.pending = false;
+    buf = it->second.buf;
+  }
+  if (wkf_device_is_planner(dev)) return;
+  unsigned long long n = 0;
+  check(wkf_buffer_download(buf.get(), 0, &n, sizeof n));
+  if (n == 0) return;
+  const unsigned long long zero = 0;
+  check(wkf_buffer_upload(buf.get(), 0, &zero, sizeof zero));
+  throw Error(WKF_ERR_HIP, "a row kernel whose blocks wait for each other gave up waiting (" + std::to_string(n) +
+                               " lanes): results computed since the last read-back are not valid");
+}
 
 TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero) {
   TensorData td;
@@ -697,8 +754,8 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   size_t nrows = 1;
   for (size_t d : out_shape) nrows *= d;
   if (nrows > 0xffffffffull) return false;
-  bool streamed = false, split = false;
-  size_t parts = 1, chunk = 0;
+  bool streamed = false, split = false, team = false;
+  size_t parts = 1, chunk = 0, teams = 0;
   if (NV > max_nv || NV * V * K > 128) {
     // The row does not fit the registers of a block.  With enough rows to occupy the chip, one block per row
     // streams its row once per stage and once more for the result, in ONE launch; the passes after the first
@@ -707,6 +764,28 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
     // of its own, which leaves its parts' values to the next (softmax: two launches).  Reductions that are
     // stored (no result rows) are folded across the whole grid by the caller instead.
     if (nvec < 1024) return false;
+    // First choice: the row in the registers of a team of blocks (one launch, one read).  Eight 16-byte vectors
+    // per lane over all operands, 256 lanes per block, at most 256 parts.  The launch bounds of the kernel
+    // guarantee four resident blocks per compute unit, and the grid never asks for more than that, because
+    // the blocks of a team wait for each other.
+    size_t kfull = 0;
+    for (size_t k = 0; k < K; k++) kfull += rb.operands[k].layout.strides[axis] == 1 ? 1 : 0;
+    const size_t team_nv = std::max<size_t>(1, 8 / std::max<size_t>(1, kfull));
+    const size_t team_lanes = 256;
+    const size_t team_parts = (nvec + team_lanes * team_nv - 1) / (team_lanes * team_nv);
+    wkf_props props;
+    check(wkf_device_props(dev_, &props));
+    const size_t resident = size_t(std::max(1, props.compute_units)) * 4;
+    // (a device that is only kept by its live buffers gets no new per-device state: the word team kernels count in)
+    if (st_.row_team && !scalars && !noalloc_ && kfull >= 1 && team_parts >= 2 && team_parts <= 256 && team_parts <= resident &&
+        !wkf_device_closing_(dev_)) {
+      team = true;
+      ragged = false;
+      T = int(team_lanes);
+      NV = team_nv;
+      parts = team_parts;
+      teams = std::min(nrows, resident / team_parts);
+    } else {
     streamed = true;
     ragged = false;
     NV = std::max<size_t>(1, std::min<size_t>(4, 8 / std::max<size_t>(1, K)));  // vectors in flight per lane and operand
@@ -721,6 +800,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
       const size_t want = std::min<size_t>(size_t(T), std::max<size_t>(1, 2048 / nrows));
       chunk = ((nvec + want - 1) / want + step - 1) / step * step;
       parts = (nvec + chunk - 1) / chunk;
+    }
     }
   }
 
@@ -738,8 +818,9 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   spec.vectors_per_lane = int(NV);
   spec.ragged = ragged;
   spec.streamed = streamed;
+  spec.team = team;
   spec.stages = rb.stages;
-  if (streamed && rb.stages.size() >= 2) {
+  if ((streamed || team) && rb.stages.size() >= 2) {
     // softmax's pair of stages, max(x) then sum(exp(x - max)), is folded in one pass over a streamed row
     const RowStage& s0 = rb.stages[0];
     const RowStage& s1 = rb.stages[1];
@@ -789,6 +870,25 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   if (ragged) d << " ragged";
   if (streamed) d << (spec.online_max_sum ? " streamed (max and sum in one pass)" : " streamed");
   const size_t rpb = size_t(spec.block / T);
+  if (team) {
+    // zero-filled slots [stages][rows][parts] of 64 bits; the device's give-up count as the last pointer
+    TensorData slots = alloc({S * nrows * parts * 2}, DType::F32, true);
+    args.ptrs.push_back(element_ptr(slots));
+    args.ptrs.push_back(team_word(dev_));
+    args.parts = to_u32(parts, "parts");
+    args.spin = st_.row_team_spin;
+    std::string sig = row_signature(spec);
+    wkf_kernel* k = kernel(sig, [&] { return row_source(spec); });
+    LaunchRecord r;
+    r.kind = "row";
+    r.signature = sig;
+    r.grid[0] = to_u32(teams * parts, "grid");
+    r.block[0] = 256;
+    d << (spec.online_max_sum ? ", max and sum in one exchange" : "") << ", rows in the registers of teams of " << parts << " blocks, " << teams << " teams";
+    r.detail = d.str();
+    record(std::move(r), k, row_pack_args(spec, args));
+    return true;
+  }
   if (!split) {
     std::string sig = row_signature(spec);
     wkf_kernel* k = kernel(sig, [&] { return row_source(spec); });

@@ -44,6 +44,8 @@ struct Settings {
   int skinny_blocks = 0;          // workgroups the decode-sized mat_mul kernels aim for; 0 = chosen (WKF_SKINNY_BLOCKS overrides)
   int reduce_unroll = 0;          // loads in flight per lane in row reduces; 0 = chosen (WKF_REDUCE_UNROLL overrides)
   bool row_split = true;             // rows too long for a block's registers and too few to stream with a block each: one launch per stage over parts of rows (WKF_ROW_SPLIT=0: fold each reduction across the grid instead)
+  bool row_team = true;              // rows too long for a block's registers that fit those of up to 256 blocks: one launch, the row read once, the blocks of a row exchange their folds and wait for each other (WKF_ROW_TEAM=0 turns it off)
+  uint32_t row_team_spin = 1u << 20; // polls a lane of such a kernel may spend waiting before it gives up (the result is then refused at read-back); top bit: part 0 stays silent (tests)
   size_t row_stream_min_rows = 256;  // fewest rows for the one-launch kernel that streams rows longer than a block's registers (WKF_ROW_STREAM_MIN_ROWS)
 };
 
@@ -54,6 +56,11 @@ struct Space {
   std::vector<size_t> shape;
   std::vector<std::vector<size_t>> strides;  // [operand][dim]
 };
+
+// Team row kernels count the lanes that gave up waiting for another block in one word per device.  Called after a
+// download has synchronised the stream: throws when the count is not zero (and clears it), so that no result of
+// such a kernel, or of anything computed from it, is handed out unnoticed.
+void team_check(wkf_device* dev);
 
 class Resolver {
  public:

@@ -164,6 +164,12 @@ void wkf_add_destroy_hook_(void (*fn)(wkf_device*)) {
 
 // The per-device scratch array of the allocation-free entry point as a buffer handle (a new reference: release it
 // like any other), and its size.  The layers above use it in place of an allocated temporary.
+// True once wkf_device_destroy has been asked for a device that buffers still keep alive.
+bool wkf_device_closing_(wkf_device* dev) {
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  return dev->closing;
+}
+
 wkf_buffer* wkf_scratch_(wkf_device* dev, size_t* bytes) {
   if (!dev || !dev->scratch_buf) return nullptr;
   if (bytes) *bytes = kScratchBytes;
@@ -268,8 +274,20 @@ int wkf_device_trim(wkf_device* dev) {
 
 static void destroy_now(wkf_device* dev);
 
+static void run_destroy_hooks(wkf_device* dev) {
+  std::vector<void (*)(wkf_device*)> hooks;
+  {
+    std::lock_guard<std::mutex> lock(g_hooks_mu);
+    hooks = g_destroy_hooks;
+  }
+  for (auto fn : hooks) fn(dev);
+}
+
 void wkf_device_destroy(wkf_device* dev) {
   if (!dev) return;
+  // the layers above drop what they keep for this device first: a buffer among that would otherwise count as live
+  // below and keep the device for good (the hooks run again, to no effect, when the device finally goes)
+  run_destroy_hooks(dev);
   {
     // Buffers (and the tensors that own them) may outlive the caller's last use of the device handle: the device
     // then lives on until the last of them is released, so that a late wkf_buffer_release / wkf_tensor_free
@@ -284,14 +302,7 @@ void wkf_device_destroy(wkf_device* dev) {
 }
 
 static void destroy_now(wkf_device* dev) {
-  {
-    std::vector<void (*)(wkf_device*)> hooks;
-    {
-      std::lock_guard<std::mutex> lock(g_hooks_mu);
-      hooks = g_destroy_hooks;
-    }
-    for (auto fn : hooks) fn(dev);
-  }
+  run_destroy_hooks(dev);
   wkf_device_trim(dev);
   for (auto& kv : dev->kernels) {
     if (kv.second->module) hipModuleUnload(kv.second->module);

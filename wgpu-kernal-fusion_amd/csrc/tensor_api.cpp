@@ -119,6 +119,7 @@ Settings settings_for(wkf_device* dev) {
     if (const char* u = getenv("WKF_MAP_TILE_VEC")) st.map_tile_vec = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_TAIL")) st.gemm_tail = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_SPLIT")) st.row_split = atoi(u) != 0;
+    if (const char* u = getenv("WKF_ROW_TEAM")) st.row_team = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_STREAM_MIN_ROWS")) st.row_stream_min_rows = size_t(std::max(1ll, atoll(u)));
     if (const char* u = getenv("WKF_SKINNY_TR_ROWS")) {
       int v = atoi(u);
@@ -458,6 +459,16 @@ int wkf_device_set_timing(wkf_device* dev, int enabled) {
     settings_for(dev);  // creates the entry (and reads the tuning knobs) on first use
     std::lock_guard<std::mutex> lock(g_settings_mu);
     g_settings[dev].timing = enabled != 0;
+  });
+}
+
+int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls) {
+  return guarded([&] {
+    need(dev, "wkf_device_set_row_teams");
+    settings_for(dev);
+    std::lock_guard<std::mutex> lock(g_settings_mu);
+    g_settings[dev].row_team = enabled != 0;
+    g_settings[dev].row_team_spin = spin_polls == 0 ? Settings().row_team_spin : spin_polls;
   });
 }
 
@@ -899,6 +910,7 @@ int wkf_tensor_as_slice_many(wkf_tensor** ts, int n, wkf_slice** out) {
       if (rc != WKF_OK) throw Error(rc, wkf_last_error());
       slices.push_back(std::move(s));
     }
+    if (n > 0) team_check(tds[0].device);
     for (int i = 0; i < n; i++) out[i] = slices[size_t(i)].release();
   });
 }
@@ -923,6 +935,7 @@ int wkf_tensor_as_slice(wkf_tensor* t, wkf_slice** out) {
     s->bytes.resize(wkf_buffer_size(td.buffer.get()));
     int rc = wkf_buffer_download(td.buffer.get(), 0, s->bytes.data(), s->bytes.size());
     if (rc != WKF_OK) throw Error(rc, wkf_last_error());
+    team_check(td.device);
     *out = s.release();
   });
 }
