@@ -785,6 +785,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
       NV = team_nv;
       parts = team_parts;
       teams = std::min(nrows, resident / team_parts);
+      teams = (nrows + (nrows + teams - 1) / teams - 1) / ((nrows + teams - 1) / teams);  // as many rounds, evenly filled
     } else {
     streamed = true;
     ragged = false;
