@@ -1184,7 +1184,7 @@ std::string row_source(const RowSpec& s) {
         o << "  if (talk_wave) {\n";
         o << "    if (t == " << XL << "u && !mute) {\n      wkf_team_put(" << slot(0, "part") << ", acc0);\n      wkf_team_put(" << slot(1, "part") << ", acc1);\n    }\n";
         o << "    float row_max = " << seed_text(ReduceOp::Max) << ", row_sum = 0.0f;\n";
-        o << "    for (u32 p = t - " << XL << "u; p < " << "a.parts" << "; p += 64u) {\n";
+        o << "    for (u32 p = t - " << XL << "u; p < a.parts; p += 64u) {\n";
         o << "      float part_max, part_sum;\n";
         o << "      wkf_team_get(" << slot(0, "p") << ", " << slot(1, "p") << ", part_max, part_sum, polls_left, gave_up);\n";
         o << "      const float m = fmaxf(part_max, row_max);\n";
