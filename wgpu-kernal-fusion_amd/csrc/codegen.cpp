@@ -1032,7 +1032,7 @@ std::string row_source(const RowSpec& s) {
     o << "typedef unsigned long long u64;\n";
     o << "static __device__ __forceinline__ void wkf_team_put(u64* slot, float v) {\n"
          "  __hip_atomic_store(slot, 0x100000000ull | (u64)__builtin_bit_cast(u32, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n}\n";
-    // up to two slots a poll (they travel together); `n` = 1 or 2
+    // two slots a poll (the loads travel together); a stage with one value passes its slot twice
     o << "static __device__ __forceinline__ void wkf_team_get(u64* slot_a, u64* slot_b, float& va, float& vb, u32& polls_left, u64* gave_up) {\n"
          "  for (;;) {\n"
          "    const u64 wa = __hip_atomic_load(slot_a, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);\n"
