@@ -832,8 +832,8 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                (32, 4096, 512), (17, 264, 1000), (8, 1000, 4096), (31, 72, 2048), (5, 4104, 136), (24, 8, 8200), (32, 1028, 700),
                # 128 x 128 tiles (products that would not fill the chip with 256 x 256 ones): full, ragged, K in slices
                (128, 128, 64), (129, 136, 64), (384, 640, 192), (200, 1000, 520), (511, 136, 2048), (33, 4096, 1024),
-               # full tiles that leave a partly filled last round on 256 compute units (272, 300 and 257 tiles): in f16 the
-               # tiles of that round run as two halves of 128 rows each
+               # full tiles that leave a partly filled last round on 256 compute units (272, 300 and 257 tiles): the
+               # tiles of that round run as two halves of 128 rows each (f16 and f32)
                (4096, 4352, 512), (2560, 7680, 1024), (256, 65792, 2048),
                # the same with ragged edges (272 and 288 tiles): a last tile row that ends inside its upper half (the lower
                # half tiles do nothing), one that ends inside its lower half, ragged columns, a K that is no multiple of 64
