@@ -856,7 +856,10 @@ def test_mat_mul(gpu, m, n, k, dtype, tol):
 
 BT_SHAPES = [(256, 512, 128), (300, 264, 2048), (100, 136, 72), (513, 260, 328), (1, 1024, 512), (7, 520, 1000),
              (32, 264, 4096), (2, 4100, 96), (20, 100, 64), (3, 5, 7), (33, 2048, 1024), (300, 1000, 515),
-             (4096, 4352, 512)]
+             (4096, 4352, 512),
+             # up to 16 rows of f32 against a transposed weight run on the vector ALUs: edge columns, a K that ends inside
+             # a step, a slice of K longer than one step
+             (12, 520, 1000), (16, 4100, 264), (9, 100, 4100), (8, 33, 8192), (1, 11008, 4096)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

@@ -494,6 +494,13 @@ def test_mat_mul_kernel_choice(wkf, planner):
     # ... and with a handful of rows W is streamed once through MFMA operands (decode)
     t = _x(wkf, planner, (2, 256), np.float16).mat_mul(w.transpose(0, 1))
     assert _kinds(t)[0] == "gemm" and "skinny B^T" in t.kernels()[0].detail and t.shape() == (2, 512)
+    # in f32 up to 16 rows take the vector ALUs instead (the f32 matrix instruction cannot keep up with the memory), more the MFMAs
+    w32 = _x(wkf, planner, (512, 256), np.float32, seed=2)
+    t = _x(wkf, planner, (16, 256), np.float32).mat_mul(w32.transpose(0, 1))
+    assert "skinny B^T valu" in t.kernels()[0].detail if _kinds(t)[0] == "gemm" else False
+    assert t.kernels()[0].signature == "gemm|gfx950|f32|skinny_bt|valu|m16|c256"
+    t = _x(wkf, planner, (17, 256), np.float32).mat_mul(w32.transpose(0, 1))
+    assert _kinds(t)[0] == "gemm" and "skinny B^T slices" in t.kernels()[0].detail
     planner.set_fusion(wkf.FUSION_REFERENCE)
     try:
         assert _kinds(_x(wkf, planner, (256, 256), np.float16).mat_mul(w.transpose(0, 1))) == ["map", "gemm"]

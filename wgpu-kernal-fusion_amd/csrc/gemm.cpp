@@ -23,6 +23,9 @@ const char* const kGemmSkinny =
 const char* const kGemmSkinnyBt =
 #include "kernels/gemm_skinny_bt.hip.inc"
     ;
+const char* const kGemmSkinnyBtF32 =
+#include "kernels/gemm_skinny_bt_f32.hip.inc"
+    ;
 const char* const kGemmSkinnyTr =
 #include "kernels/gemm_skinny_tr.hip.inc"
     ;
@@ -203,17 +206,28 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     const size_t gridx = (N + 127) / 128;
     // workgroups to aim for, from a sweep on MI355X ([M x 4096] x W[11008 x 4096]^T and W[4096 x 4096]^T): more slices
     // fill the chip, fewer keep the f32 partial sums (written and read once more by the fold) small as M grows
+    // up to 16 rows of f32: the vector ALUs keep up with the memory where the f32 matrix instruction (on 32 padded
+    // rows) does not; the block keeps its slice of A in the LDS, which bounds the slice
+    // ([M x 4096] x W[11008 x 4096]^T, kernel + fold: M = 1 54 -> 34 us, M = 8 58 -> 43, M = 16 71 -> 61; [16 x 11008] x W[4096 x 11008]^T 65 -> 44)
+    const bool valu = a.dtype == DType::F32 && M <= 16;
     const size_t want = st_.skinny_blocks > 0 ? size_t(st_.skinny_blocks) : (M >= 16 ? 512 : 1024);
     size_t S = (want + gridx * batch - 1) / (gridx * batch);
     S = std::min(S, std::max<size_t>(1, K * dtype_size(a.dtype) / (8 * M)));  // partial sums stay under half of W's bytes
     S = std::min(S, std::max<size_t>(1, K / (2 * kblock)));
+    if (valu) S = std::max(S, (K + 2047) / 2048);
     size_t chunk = (K + S - 1) / S;
     chunk = (chunk + kblock - 1) / kblock * kblock;
     S = (K + chunk - 1) / chunk;
     if (S > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many K slices");
     TensorData part = alloc(slices_shape(S), DType::F32, false);
-    const std::string sig = std::string("gemm|gfx950|") + dtype_name(a.dtype) + "|skinny_bt|mfma32x32";
-    wkf_kernel* k = kernel(sig, [&] { return std::string("#define WKF_H ") + (a.dtype == DType::F16 ? "1" : "0") + "\n" + kGemmSkinnyBt; });
+    size_t chunk_max = 256;
+    while (chunk_max < chunk) chunk_max *= 2;
+    const std::string sig = valu ? "gemm|gfx950|f32|skinny_bt|valu|m" + std::to_string(M) + "|c" + std::to_string(chunk_max)
+                                 : std::string("gemm|gfx950|") + dtype_name(a.dtype) + "|skinny_bt|mfma32x32";
+    wkf_kernel* k = kernel(sig, [&] {
+      if (valu) return "#define WKF_M " + std::to_string(M) + "\n#define WKF_CHUNK_MAX " + std::to_string(chunk_max) + "\n" + kGemmSkinnyBtF32;
+      return std::string("#define WKF_H ") + (a.dtype == DType::F16 ? "1" : "0") + "\n" + kGemmSkinnyBt;
+    });
     struct {
       const void* a;
       const void* w;
@@ -231,7 +245,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.grid[1] = uint32_t(S);
     r.grid[2] = uint32_t(batch);
     std::ostringstream d;
-    d << "m=" << M << " n=" << N << " k=" << K << " skinny B^T slices=" << S;
+    d << "m=" << M << " n=" << N << " k=" << K << " skinny B^T" << (valu ? " valu" : "") << " slices=" << S;
     if (batch > 1) d << " batch=" << batch;
     r.detail = d.str();
     record(std::move(r), k, sbytes);
