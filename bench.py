@@ -336,6 +336,16 @@ def build_workloads(w, dev, seeded, which, with_cpu=False):
         bm_ = T.new(dev, seeded(7, 7, (4096, 11008), "normal", dtype=F16, std=0.02))
         out["more_gemm_mid"] = Workload("512 rows against a wide weight: GEMM f16 [512x4096]x[4096x11008]", [[am_.mat_mul(bm_)]],
                                         2 * 512 * 4096 * 11008, "TFLOP/s", F16_MFMA_PEAK_TFLOPS, "f16")
+    if "decode" in which:
+        # one row against a transposed weight (x . W^T, the linear layer at decode time; no BASELINE configuration): reading
+        # W once is all the work, so the product is priced against HBM.  Three weights take turns, more bytes than
+        # the last-level cache holds.
+        for name, dt, key in (("f16", np.float16, "decode_f16"), ("f32", np.float32, "decode_f32")):
+            xr = T.new(dev, seeded(8, 0, (1, 4096), "normal", dtype=dt))
+            ws = [T.new(dev, seeded(8, 1 + r, (11008, 4096), "normal", dtype=dt, std=0.02)) for r in range(4 if dt == np.float16 else 3)]
+            esz = 2 if dt == np.float16 else 4
+            out[key] = Workload(f"decode: x.W^T, {name} [1x4096]x[11008x4096]^T", [[xr.mat_mul(w_.transpose(0, 1))] for w_ in ws],
+                                (11008 * 4096 + 4096 + 11008) * esz, "GB/s", HBM_PEAK_GBS, name)
     if "long" in which:
         # rows longer than a block's registers (no BASELINE configuration; the reference's reduce takes any length)
         xs = [T.new(dev, seeded(4, 40 + r, (256, 262144), "normal")) for r in range(2)]
@@ -434,7 +444,7 @@ def cpu_baseline(wl):
                       "oracle/port.c with OpenMP"}
 
 
-GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16", "long", "attn", "more")
+GROUPS = ("c1", "c2", "c3", "c4", "c5", "f16", "long", "attn", "more", "decode")
 
 
 def plan_only(w):
@@ -703,7 +713,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-detail", action="store_true", help="only the headline configuration")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baselines")
-    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16,long,attn,more for the detail table")
+    ap.add_argument("--only", default="", help="comma-separated subset of c1,c2,c3,c4,c5,f16,long,attn,more,decode for the detail table")
     ap.add_argument("--plan-only", action="store_true",
                     help="no GPU: plan every workload on a plan-only device so that each kernel is JIT-compiled into the cache")
     ap.add_argument("--profile", default="", help="run one workload only (copy, c1, c2a, c2b, c3, c4_rmsnorm, c4_rope, c4_softmax, "

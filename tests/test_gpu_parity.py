@@ -859,7 +859,9 @@ BT_SHAPES = [(256, 512, 128), (300, 264, 2048), (100, 136, 72), (513, 260, 328),
              (4096, 4352, 512),
              # up to 16 rows of f32 against a transposed weight run on the vector ALUs: edge columns, a K that ends inside
              # a step, a slice of K longer than one step
-             (12, 520, 1000), (16, 4100, 264), (9, 100, 4100), (8, 33, 8192), (1, 11008, 4096)]
+             (12, 520, 1000), (16, 4100, 264), (9, 100, 4100), (8, 33, 8192), (1, 11008, 4096),
+             # f16: up to 4 rows; rows of A that fit the LDS whole take one launch with 2, 4 or 8 rows of W a wave
+             (3, 1000, 520), (4, 4100, 136), (2, 100, 4104), (1, 33, 8200), (4, 20000, 64), (2, 6000, 12296)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])
@@ -891,6 +893,7 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 # starts its walk over K at a different tile and wraps around; K with a partial last tile, B^T, edge columns
                 ((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False)]
 # many full tiles over K = 64 or 128: one workgroup per compute unit walks the tiles of the whole batch
+BATCH_SHAPES += [((5,), 2, 300, 264, True), ((40,), 1, 1000, 72, True), ((2, 3), 4, 260, 4096, True)]  # decode rows on the vector ALUs
 BATCH_SHAPES += [((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)]
 WHOLE_K = {((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)}
 ROTATED = {((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False),

@@ -497,8 +497,11 @@ def test_mat_mul_kernel_choice(wkf, planner):
     # in f32 up to 16 rows take the vector ALUs instead (the f32 matrix instruction cannot keep up with the memory), more the MFMAs
     w32 = _x(wkf, planner, (512, 256), np.float32, seed=2)
     t = _x(wkf, planner, (16, 256), np.float32).mat_mul(w32.transpose(0, 1))
-    assert "skinny B^T valu" in t.kernels()[0].detail if _kinds(t)[0] == "gemm" else False
-    assert t.kernels()[0].signature == "gemm|gfx950|f32|skinny_bt|valu|m16|c256"
+    # (rows of A that fit the LDS whole: one launch, no K slices; here 16 x 256 floats; a wave walks one row of W)
+    assert _kinds(t) == ["gemm"] and t.kernels()[0].detail.endswith("skinny B^T valu whole K, 1 rows a wave")
+    assert t.kernels()[0].signature == "gemm|gfx950|f32|skinny_bt|valu|m16|c1024|r1"
+    big = _x(wkf, planner, (16, 4096), np.float32).mat_mul(_x(wkf, planner, (512, 4096), np.float32, seed=2).transpose(0, 1))
+    assert len(_kinds(big)) == 2 and "skinny B^T valu slices=" in big.kernels()[0].detail  # 256 KiB of A: K in slices, then the fold
     t = _x(wkf, planner, (17, 256), np.float32).mat_mul(w32.transpose(0, 1))
     assert _kinds(t)[0] == "gemm" and "skinny B^T slices" in t.kernels()[0].detail
     planner.set_fusion(wkf.FUSION_REFERENCE)
@@ -526,8 +529,11 @@ def test_batched_mat_mul_is_one_launch(wkf, planner):
     q1 = _x(wkf, planner, (8, 1, 128), np.float16, seed=3)
     kv = _x(wkf, planner, (8, 2048, 128), np.float16, seed=4)
     s1 = q1.mat_mul(kv.transpose(1, 2))
-    assert _kinds(s1)[0] == "gemm" and len(_kinds(s1)) == 2           # the product, then the fold over the K slices
-    assert "skinny B^T" in s1.kernels()[0].detail and s1.kernels()[0].detail.endswith("batch=8")
+    # (one launch: the vector-ALU kernel for one row of f16 folds its K slices itself, the last wave to finish 32 rows)
+    assert _kinds(s1) == ["gemm"]
+    assert "skinny B^T valu" in s1.kernels()[0].detail and s1.kernels()[0].detail.endswith("batch=8")
+    s8 = _x(wkf, planner, (8, 8, 128), np.float16, seed=3).mat_mul(kv.transpose(1, 2))
+    assert _kinds(s8)[0] == "gemm" and len(_kinds(s8)) == 2 and "skinny B^T slices" in s8.kernels()[0].detail  # more rows: MFMAs, then the fold
     o1 = s1.mat_mul(kv)
     assert o1.shape() == (8, 1, 128) and _kinds(o1)[-2:] == ["gemm", "red_col"]
     assert "skinny slices" in o1.kernels()[-2].detail and o1.kernels()[-2].detail.endswith("batch=8")

@@ -23,8 +23,8 @@ const char* const kGemmSkinny =
 const char* const kGemmSkinnyBt =
 #include "kernels/gemm_skinny_bt.hip.inc"
     ;
-const char* const kGemmSkinnyBtF32 =
-#include "kernels/gemm_skinny_bt_f32.hip.inc"
+const char* const kGemmSkinnyBtValu =
+#include "kernels/gemm_skinny_bt_valu.hip.inc"
     ;
 const char* const kGemmSkinnyTr =
 #include "kernels/gemm_skinny_tr.hip.inc"
@@ -209,23 +209,42 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     // up to 16 rows of f32: the vector ALUs keep up with the memory where the f32 matrix instruction (on 32 padded
     // rows) does not; the block keeps its slice of A in the LDS, which bounds the slice
     // ([M x 4096] x W[11008 x 4096]^T, kernel + fold: M = 1 54 -> 34 us, M = 8 58 -> 43, M = 16 71 -> 61; [16 x 11008] x W[4096 x 11008]^T 65 -> 44)
-    const bool valu = a.dtype == DType::F32 && M <= 16;
+    const bool valu = a.dtype == DType::F32 ? M <= 16 : M <= 4;
     const size_t want = st_.skinny_blocks > 0 ? size_t(st_.skinny_blocks) : (M >= 16 ? 512 : 1024);
     size_t S = (want + gridx * batch - 1) / (gridx * batch);
     S = std::min(S, std::max<size_t>(1, K * dtype_size(a.dtype) / (8 * M)));  // partial sums stay under half of W's bytes
     S = std::min(S, std::max<size_t>(1, K / (2 * kblock)));
-    if (valu) S = std::max(S, (K + 2047) / 2048);
+    if (valu) S = std::max(S, (K + 2047) / 2048);  // the LDS holds at most 2048 elements of each row of A
     size_t chunk = (K + S - 1) / S;
     chunk = (chunk + kblock - 1) / kblock * kblock;
     S = (K + chunk - 1) / chunk;
     if (S > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many K slices");
-    TensorData part = alloc(slices_shape(S), DType::F32, false);
+    // Rows of A that fit the LDS whole: no slices and no second launch
+    // ([1 x 4096] x W[11008 x 4096]^T f16: 16.8 + 3.9 us in two launches -> 14.6 us in one; f32: 31.9 + 4.0 -> 29.6)
+    const size_t vlen = 16 / dtype_size(a.dtype);
+    const size_t k_lds = (K + 256 * vlen - 1) / (256 * vlen) * (256 * vlen);
+    const bool whole_k = valu && M * k_lds * dtype_size(a.dtype) <= 65536;
+    // (a whole wave walks one row of W, 1 KiB a load, unless a row is shorter than that: measured on
+    // [1 x 4096] x W[11008 x 4096]^T with 1, 2, 4, 8 rows a wave, f16 14.6, 18.5, 15.7, 20.2 us, f32 29.6, 30.3, 38.4, 33.9 us)
+    size_t rows_per_wave = 1;
+    while (rows_per_wave < 8 && K * dtype_size(a.dtype) * rows_per_wave < 1024) rows_per_wave *= 2;
+    if (whole_k) {
+      S = 1;
+      chunk = K;
+    }
+    TensorData part = whole_k ? TensorData() : alloc(slices_shape(S), DType::F32, false);
+    TensorData out_whole = whole_k ? alloc(out_shape, a.dtype, false) : TensorData();
     size_t chunk_max = 256;
     while (chunk_max < chunk) chunk_max *= 2;
-    const std::string sig = valu ? "gemm|gfx950|f32|skinny_bt|valu|m" + std::to_string(M) + "|c" + std::to_string(chunk_max)
+    if (whole_k) chunk_max = k_lds;
+    const std::string sig = valu ? std::string("gemm|gfx950|") + dtype_name(a.dtype) + "|skinny_bt|valu|m" + std::to_string(M) + "|c" + std::to_string(chunk_max) +
+                                       (whole_k ? "|r" + std::to_string(rows_per_wave) : std::string())
                                  : std::string("gemm|gfx950|") + dtype_name(a.dtype) + "|skinny_bt|mfma32x32";
     wkf_kernel* k = kernel(sig, [&] {
-      if (valu) return "#define WKF_M " + std::to_string(M) + "\n#define WKF_CHUNK_MAX " + std::to_string(chunk_max) + "\n" + kGemmSkinnyBtF32;
+      if (valu)
+        return std::string("#define WKF_H ") + (a.dtype == DType::F16 ? "1" : "0") + "\n#define WKF_M " + std::to_string(M) + "\n#define WKF_CHUNK_MAX " +
+               std::to_string(chunk_max) + "\n#define WKF_WHOLE_K " + (whole_k ? "1" : "0") + "\n#define WKF_R " + std::to_string(rows_per_wave) + "\n" +
+               kGemmSkinnyBtValu;
       return std::string("#define WKF_H ") + (a.dtype == DType::F16 ? "1" : "0") + "\n" + kGemmSkinnyBt;
     });
     struct {
@@ -233,22 +252,36 @@ TensorData Resolver::run_matmul(const NodeP& n) {
       const void* w;
       void* part;
       uint32_t m, n, k, chunk;
-    } sargs = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(part.buffer.get()),
+    } sargs = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), whole_k ? nullptr : wkf_buffer_ptr(part.buffer.get()),
                uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(chunk)};
     std::vector<unsigned char> sbytes(sizeof(sargs));
     memcpy(sbytes.data(), &sargs, sizeof(sargs));
+    if (valu) {
+      struct {
+        const void* a;
+        const void* w;
+        void* part;
+        void* c;
+        uint32_t m, n, k, chunk;
+      } vargs = {sargs.a, sargs.w, sargs.part, whole_k ? wkf_buffer_ptr(out_whole.buffer.get()) : nullptr, sargs.m, sargs.n, sargs.k, sargs.chunk};
+      sbytes.resize(sizeof(vargs));
+      memcpy(sbytes.data(), &vargs, sizeof(vargs));
+    }
     LaunchRecord r;
     r.kind = "gemm";
     r.signature = sig;
     r.block[0] = 256;
-    r.grid[0] = uint32_t(gridx);
+    r.grid[0] = uint32_t(whole_k ? (N + 4 * rows_per_wave - 1) / (4 * rows_per_wave) : gridx);
     r.grid[1] = uint32_t(S);
     r.grid[2] = uint32_t(batch);
     std::ostringstream d;
-    d << "m=" << M << " n=" << N << " k=" << K << " skinny B^T" << (valu ? " valu" : "") << " slices=" << S;
+    d << "m=" << M << " n=" << N << " k=" << K << " skinny B^T" << (valu ? " valu" : "");
+    if (whole_k) d << " whole K, " << rows_per_wave << " rows a wave";
+    else d << " slices=" << S;
     if (batch > 1) d << " batch=" << batch;
     r.detail = d.str();
     record(std::move(r), k, sbytes);
+    if (whole_k) return out_whole;
     return fold_slices(part);
   }
   // Up to 32 rows of A against a row-major f16 B: B is streamed once through wave-private LDS tiles and read back
