@@ -824,6 +824,8 @@ GEMM_SHAPES = [(1, 1, 1), (2, 2, 1), (3, 5, 7), (17, 33, 65), (64, 64, 64), (100
                # few tiles over a long K: K is cut into slices across the grid (f32 partial sums + a reduce)
                (300, 264, 2048), (128, 1032, 4096), (512, 512, 8192), (256, 256, 2048), (40, 512, 1096),
                (1, 1024, 512), (5, 2048, 300), (16, 520, 1000), (8, 264, 4096), (2, 96, 8192), (3, 4104, 77),
+               # ... and against a narrow B (rows of at most 2 KiB): the lanes of a block share consecutive rows of B
+               (1, 128, 2048), (4, 1000, 515), (3, 8, 70000), (1, 64, 1100), (2, 1024, 64),
                # rows of B off the 16-byte grid (N odd): a transposed copy of B keeps a large product on the MFMA kernels
                (300, 1001, 512), (512, 1002, 256), (17, 1003, 4096), (1, 5001, 4096),
                # K off the vector grid: zero-padded copies of A and B keep a large product on the MFMA kernels
@@ -893,6 +895,7 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
                 # starts its walk over K at a different tile and wraps around; K with a partial last tile, B^T, edge columns
                 ((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False)]
 # many full tiles over K = 64 or 128: one workgroup per compute unit walks the tiles of the whole batch
+BATCH_SHAPES += [((3,), 4, 72, 300, False), ((64,), 1, 64, 1024, False)]  # decode rows against a narrow B
 BATCH_SHAPES += [((5,), 2, 300, 264, True), ((40,), 1, 1000, 72, True), ((2, 3), 4, 260, 4096, True)]  # decode rows on the vector ALUs
 BATCH_SHAPES += [((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)]
 WHOLE_K = {((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)}

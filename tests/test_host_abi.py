@@ -536,7 +536,9 @@ def test_batched_mat_mul_is_one_launch(wkf, planner):
     assert _kinds(s8)[0] == "gemm" and len(_kinds(s8)) == 2 and "skinny B^T slices" in s8.kernels()[0].detail  # more rows: MFMAs, then the fold
     o1 = s1.mat_mul(kv)
     assert o1.shape() == (8, 1, 128) and _kinds(o1)[-2:] == ["gemm", "red_col"]
-    assert "skinny slices" in o1.kernels()[-2].detail and o1.kernels()[-2].detail.endswith("batch=8")
+    # (128 columns: a narrow B, whose rows the lanes of a block share among themselves)
+    assert "skinny narrow slices" in o1.kernels()[-2].detail and o1.kernels()[-2].detail.endswith("batch=8")
+    assert o1.kernels()[-2].signature.endswith("|skinny|m1|v8|narrow16")
     # the same binaries as a single product: no new module for the batch
     before = planner.module_stats()
     _x(wkf, planner, (3, 256, 64), np.float16).mat_mul(_x(wkf, planner, (3, 64, 256), np.float16, seed=1)).materialize()

@@ -20,6 +20,9 @@ const char* const kGemmGeneric =
 const char* const kGemmSkinny =
 #include "kernels/gemm_skinny.hip.inc"
     ;
+const char* const kGemmSkinnyNarrow =
+#include "kernels/gemm_skinny_narrow.hip.inc"
+    ;
 const char* const kGemmSkinnyBt =
 #include "kernels/gemm_skinny_bt.hip.inc"
     ;
@@ -331,11 +334,17 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // across the grid, then one reduce launch that adds the slices and rounds to the tensor dtype.
   if (st_.fusion == FusionMode::Tree && !bt && M <= (a.dtype == DType::F16 ? kSkinnyRowsF16 : kSkinnyRowsF32) && N % V == 0 && K >= 16 && N * K >= (size_t(1) << 16)) {
     const size_t esize = dtype_size(a.dtype);
-    const size_t colblocks = (N + 256 * V - 1) / (256 * V);
+    // A narrow B (rows of at most 2 KiB, p . v at decode time) would leave most lanes of the lane-per-column kernel
+    // without columns: its lanes cover a few consecutive rows of B each instead
+    // ([32,1,2048] x [32,2048,128] f16: 11.5 -> 3 us before the fold)
+    const bool narrow = M <= 4 && N / V <= 128 && K >= 64;
+    size_t lanes_per_row = 1;
+    while (lanes_per_row < N / V) lanes_per_row *= 2;
+    const size_t colblocks = narrow ? 1 : (N + 256 * V - 1) / (256 * V);
     const size_t want = st_.skinny_blocks > 0 ? size_t(st_.skinny_blocks) : 1024;
     size_t S = (want + colblocks * batch - 1) / (colblocks * batch);
     S = std::min(S, std::max<size_t>(1, K * esize / (8 * M)));  // partial sums stay under half of B's bytes
-    S = std::min(S, K / 16);
+    S = std::min(S, K / (narrow ? 64 : 16));
     S = std::max<size_t>(S, 1);
     size_t chunk = (K + S - 1) / S;
     chunk = (chunk + 3) & ~size_t(3);
@@ -344,11 +353,13 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     TensorData part = alloc(slices_shape(S), DType::F32, false);
     std::ostringstream sg;
     sg << "gemm|gfx950|" << dtype_name(a.dtype) << "|skinny|m" << M << "|v" << V;
+    if (narrow) sg << "|narrow" << lanes_per_row;
     const std::string sig = sg.str();
     wkf_kernel* k = kernel(sig, [&] {
       std::ostringstream src;
-      src << "#define WKF_T " << (a.dtype == DType::F32 ? "float" : "_Float16") << "\n#define WKF_V " << V << "\n#define WKF_M " << M
-          << "\n" << kGemmSkinny;
+      src << "#define WKF_T " << (a.dtype == DType::F32 ? "float" : "_Float16") << "\n#define WKF_V " << V << "\n#define WKF_M " << M << "\n";
+      if (narrow) src << "#define WKF_LR " << lanes_per_row << "\n" << kGemmSkinnyNarrow;
+      else src << kGemmSkinny;
       return src.str();
     });
     struct {
@@ -368,7 +379,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     r.grid[1] = uint32_t(S);
     r.grid[2] = uint32_t(batch);
     std::ostringstream d;
-    d << "m=" << M << " n=" << N << " k=" << K << " skinny slices=" << S;
+    d << "m=" << M << " n=" << N << " k=" << K << " skinny" << (narrow ? " narrow" : "") << " slices=" << S;
     if (batch > 1) d << " batch=" << batch;
     r.detail = d.str();
     record(std::move(r), k, sbytes);
