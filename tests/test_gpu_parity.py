@@ -856,6 +856,24 @@ def test_mat_mul(gpu, m, n, k, dtype, tol):
     gemm_check(got, a, b, tol)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+@pytest.mark.parametrize("m,n,k,bt", [(1, 128, 1024, False), (2, 64, 3000, False), (1, 4096, 520, False), (1, 300, 4096, True),
+                                      (8, 100, 8192, True), (3, 1000, 264, True), (40, 264, 512, False), (300, 264, 136, True)],
+                         ids=lambda v: str(v))
+def test_mat_mul_with_an_infinite_operand_has_no_stray_nan(gpu, m, n, k, bt, dtype):
+    # Kernels pad with zeros past the end of K, of a slice of K or of a tile, and zero times an infinite operand
+    # would be NaN: with a positive B and +inf in the last (and the first) column of A every product is +inf.
+    rng = np.random.default_rng(m * 31 + n * 7 + k)
+    a = rng.uniform(0.5, 1.0, (m, k)).astype(dtype)
+    b = rng.uniform(0.5, 1.0, (n, k) if bt else (k, n)).astype(dtype)
+    a[:, k - 1] = np.inf
+    a[0, 0] = np.inf
+    api = HipAPI(gpu)
+    tb = api.tensor(b)
+    got = hip_values(api.tensor(a).mat_mul(tb.transpose(0, 1) if bt else tb))
+    assert got.shape == (m, n) and np.all(np.isposinf(got)), (np.isnan(got).sum(), np.isfinite(got).sum())
+
+
 BT_SHAPES = [(256, 512, 128), (300, 264, 2048), (100, 136, 72), (513, 260, 328), (1, 1024, 512), (7, 520, 1000),
              (32, 264, 4096), (2, 4100, 96), (20, 100, 64), (3, 5, 7), (33, 2048, 1024), (300, 1000, 515),
              (4096, 4352, 512),
