@@ -860,14 +860,23 @@ def test_mat_mul(gpu, m, n, k, dtype, tol):
 @pytest.mark.parametrize("m,n,k,bt", [(1, 128, 1024, False), (2, 64, 3000, False), (1, 4096, 520, False), (1, 300, 4096, True),
                                       (8, 100, 8192, True), (3, 1000, 264, True), (40, 264, 512, False), (300, 264, 136, True)],
                          ids=lambda v: str(v))
-def test_mat_mul_with_an_infinite_operand_has_no_stray_nan(gpu, m, n, k, bt, dtype):
+@pytest.mark.parametrize("side", ["a", "b"])
+def test_mat_mul_with_an_infinite_operand_has_no_stray_nan(gpu, m, n, k, bt, dtype, side):
     # Kernels pad with zeros past the end of K, of a slice of K or of a tile, and zero times an infinite operand
-    # would be NaN: with a positive B and +inf in the last (and the first) column of A every product is +inf.
+    # would be NaN: with positive operands and +inf in the last (and the first) position along K of A, or of B, every
+    # product is +inf.
     rng = np.random.default_rng(m * 31 + n * 7 + k)
     a = rng.uniform(0.5, 1.0, (m, k)).astype(dtype)
     b = rng.uniform(0.5, 1.0, (n, k) if bt else (k, n)).astype(dtype)
-    a[:, k - 1] = np.inf
-    a[0, 0] = np.inf
+    if side == "a":
+        a[:, k - 1] = np.inf
+        a[0, 0] = np.inf
+    elif bt:
+        b[:, k - 1] = np.inf
+        b[n - 1, 0] = np.inf
+    else:
+        b[k - 1, :] = np.inf
+        b[0, n - 1] = np.inf
     api = HipAPI(gpu)
     tb = api.tensor(b)
     got = hip_values(api.tensor(a).mat_mul(tb.transpose(0, 1) if bt else tb))
