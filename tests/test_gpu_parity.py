@@ -890,7 +890,10 @@ BT_SHAPES = [(256, 512, 128), (300, 264, 2048), (100, 136, 72), (513, 260, 328),
              # a step, a slice of K longer than one step
              (12, 520, 1000), (16, 4100, 264), (9, 100, 4100), (8, 33, 8192), (1, 11008, 4096),
              # f16: up to 4 rows; rows of A that fit the LDS whole take one launch with 2, 4 or 8 rows of W a wave
-             (3, 1000, 520), (4, 4100, 136), (2, 100, 4104), (1, 33, 8200), (4, 20000, 64), (2, 6000, 12296)]
+             (3, 1000, 520), (4, 4100, 136), (2, 100, 4104), (1, 33, 8200), (4, 20000, 64), (2, 6000, 12296),
+             # 5 to 16 rows against at least 256 groups of 32 rows of W: the eight waves of a block share K (edge rows
+             # of W, a K that leaves some waves without work, a K that ends inside a step)
+             (8, 8200, 1024), (16, 9000, 520), (5, 8192, 4104), (12, 10000, 8192)]
 
 
 @pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-3), (np.float16, 1e-2)], ids=["f32", "f16"])

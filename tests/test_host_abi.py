@@ -502,6 +502,9 @@ def test_mat_mul_kernel_choice(wkf, planner):
     assert t.kernels()[0].signature == "gemm|gfx950|f32|skinny_bt|valu|m16|c1024|r1"
     big = _x(wkf, planner, (16, 4096), np.float32).mat_mul(_x(wkf, planner, (512, 4096), np.float32, seed=2).transpose(0, 1))
     assert len(_kinds(big)) == 2 and "skinny B^T valu slices=" in big.kernels()[0].detail  # 256 KiB of A: K in slices, then the fold
+    # 5 to 16 rows of f16 against enough rows of W to give every compute unit a block: one launch, the eight waves of a block share K
+    wide16 = _x(wkf, planner, (8, 1024), np.float16).mat_mul(_x(wkf, planner, (8192, 1024), np.float16, seed=2).transpose(0, 1))
+    assert _kinds(wide16) == ["gemm"] and wide16.kernels()[0].detail.endswith("skinny B^T, K over the 8 waves of a block")
     t = _x(wkf, planner, (17, 256), np.float32).mat_mul(w32.transpose(0, 1))
     assert _kinds(t)[0] == "gemm" and "skinny B^T slices" in t.kernels()[0].detail
     planner.set_fusion(wkf.FUSION_REFERENCE)

@@ -26,6 +26,9 @@ const char* const kGemmSkinnyNarrow =
 const char* const kGemmSkinnyBt =
 #include "kernels/gemm_skinny_bt.hip.inc"
     ;
+const char* const kGemmSkinnyBtBlock =
+#include "kernels/gemm_skinny_bt_block.hip.inc"
+    ;
 const char* const kGemmSkinnyBtValu =
 #include "kernels/gemm_skinny_bt_valu.hip.inc"
     ;
@@ -206,6 +209,41 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   };
   if (skinny_bt) {
     const size_t kblock = 128 / dtype_size(a.dtype);  // 128 bytes of every row per step
+    const bool valu_rows = a.dtype == DType::F32 ? M <= 16 : M <= 4;
+    wkf_props bprops;
+    if (wkf_device_props(dev_, &bprops) != WKF_OK) throw Error(WKF_ERR_HIP, wkf_last_error());
+    if (!valu_rows && M <= 16 && (N + 31) / 32 * batch >= size_t(std::max(1, bprops.compute_units)) && K >= 8 * kblock) {
+      // Enough groups of 32 rows of W to give every compute unit a block: the eight waves of a block share K among
+      // themselves and add up through the LDS, so there are no partial sums in memory and no second launch
+      // ([M x 4096] x W[11008 x 4096]^T f16, M = 8: 22.4 + 4.0 us -> 25.0 us, M = 16: 27.9 + 4.0 -> 27.2; at M = 32 the
+      // short walks of K cost more than the second launch)
+      size_t chunk = (K + 7) / 8;
+      chunk = (chunk + kblock - 1) / kblock * kblock;
+      TensorData out = alloc(out_shape, a.dtype, false);
+      const std::string sig = std::string("gemm|gfx950|") + dtype_name(a.dtype) + "|skinny_bt|mfma32x32|block8";
+      wkf_kernel* k = kernel(sig, [&] { return std::string("#define WKF_H ") + (a.dtype == DType::F16 ? "1" : "0") + "\n" + kGemmSkinnyBtBlock; });
+      struct {
+        const void* a;
+        const void* w;
+        void* c;
+        uint32_t m, n, k, chunk;
+      } bargs = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(out.buffer.get()),
+                 uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(chunk)};
+      std::vector<unsigned char> bbytes(sizeof(bargs));
+      memcpy(bbytes.data(), &bargs, sizeof(bargs));
+      LaunchRecord r;
+      r.kind = "gemm";
+      r.signature = sig;
+      r.block[0] = 512;
+      r.grid[0] = uint32_t((N + 31) / 32);
+      r.grid[2] = uint32_t(batch);
+      std::ostringstream d;
+      d << "m=" << M << " n=" << N << " k=" << K << " skinny B^T, K over the 8 waves of a block";
+      if (batch > 1) d << " batch=" << batch;
+      r.detail = d.str();
+      record(std::move(r), k, bbytes);
+      return out;
+    }
     const size_t gridx = (N + 127) / 128;
     // workgroups to aim for, from a sweep on MI355X ([M x 4096] x W[11008 x 4096]^T and W[4096 x 4096]^T): more slices
     // fill the chip, fewer keep the f32 partial sums (written and read once more by the fold) small as M grows
