@@ -11,7 +11,9 @@ GB/s of the whole step by the wall clock, inputs resident in HBM, steps rotating
 over several input tensors so that the 256 MB Infinity Cache cannot serve them.
 `roofline` is the dominant kernel (the exp-sum reduce) timed with hipEvent pairs
 on the stream it runs on; `cpu_baseline` is the CPU port of the reference's
-decomposition (oracle/port.c) on this box's host cores; `all_configs` carries
+decomposition (oracle/port.c) on this box's host cores; the line also carries `fracs`, one
+[fraction of roofline, microseconds per step] pair per configuration, and stays below 4 KB.  The rows behind it
+(`all_configs`) are written to the file `--detail-out` names:
 every BASELINE configuration (GB/s or TFLOP/s, the fraction of its roofline, the median and the minimum of the
 per-launch times after at least 100 warm launches, and the CPU port timed on a bounded sample of the same
 configuration), plus f16 rows of the memory-bound kernels.
@@ -706,6 +708,38 @@ def yardsticks(w, dev, seeded, which, launches):
     print(json.dumps(out))
 
 
+MAX_LINE_BYTES = 4096  # the final stdout line must stay small enough for any reader of it to parse
+
+
+def final_line(result):
+    """(the ONE stdout line, the full record).  The line keeps the contract keys, `roofline`, `cpu_baseline`, the
+    worst BASELINE configuration and one [fraction of roofline, back-to-back us per step] pair per configuration;
+    the rows themselves (kernels, medians, CPU samples) are in the full record only."""
+    full = dict(result)
+    detail = full.get("all_configs") or []
+    if detail:
+        # the configuration furthest below its roofline (BASELINE configurations only, as this library fuses them)
+        own = [r for r in detail if r["key"][0] == "c" and not r["key"].endswith("_reference_rules") and r["key"] != "c2_one_pass"]
+        if own:
+            worst = min(own, key=lambda r: r["roofline"]["frac"])
+            full["worst_config"] = {"key": worst["key"], "name": worst["name"], "frac": worst["roofline"]["frac"],
+                                    "achieved": worst["roofline"]["achieved"], "unit": worst["unit"]}
+    line = {k: v for k, v in full.items() if k != "all_configs"}
+    ref = line.get("reference_cpu_path")
+    if isinstance(ref, dict):
+        line["reference_cpu_path"] = {"available": ref.get("available"), "note": ref.get("note")}
+    if detail:
+        line["fracs"] = {r["key"]: [r["roofline"]["frac"], r["roofline"]["avg_us"]] for r in detail}
+    text = json.dumps(line, separators=(",", ":"))
+    if len(text) > MAX_LINE_BYTES:  # never grow past the limit: drop the optional parts, longest first
+        for k in ("reference_cpu_path", "fracs"):
+            line.pop(k, None)
+            text = json.dumps(line, separators=(",", ":"))
+            if len(text) <= MAX_LINE_BYTES:
+                break
+    return text, full
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -720,6 +754,8 @@ def main():
                                                   "c5_f32, c5_f16, c5_mlp, f16_*), for a profiler")
     ap.add_argument("--launches", type=int, default=30, help="timed steps of --profile / launches of --yardstick mfma")
     ap.add_argument("--warm-ms", type=float, default=300.0, help="--profile: milliseconds of untimed steps before the timed ones")
+    ap.add_argument("--detail-out", default="gpurun_out/bench_detail.json",
+                    help="file (relative to this one) that receives the full record with every row; empty: none")
     ap.add_argument("--yardstick", default="", help="mfma | stream: bounds of the machine measured with kernels outside the library")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -774,8 +810,7 @@ def main():
                    "device": props.arch.decode(), "compute_units": props.compute_units, "clock_khz": props.clock_khz},
         "roofline": {"bound": "hbm", "achieved": round(268468224 / dominant["us"] * 1e-3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(268468224 / dominant["us"] * 1e-3 / HBM_PEAK_GBS, 4), "traffic": traffic,
-                     "traffic_source": "profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel, calibrated "
-                                       "with the copy kernel, taken in a profiler run of its own; not measured by this run",
+                     "traffic_source": "profiles/traffic.json (rocprofv3 --pmc run of this kernel, calibrated with a copy kernel; not measured by this run)",
                      "kernel": dominant["kind"] + " " + dominant["detail"], "avg_us": dominant["us"],
                      "algorithmic_bytes_per_launch": 268468224},
         "value_frac_of_hbm_peak": round(value / HBM_PEAK_GBS, 4),
@@ -821,13 +856,13 @@ def main():
             del wls
             dev.trim()
         result["all_configs"] = detail
-        # the configuration furthest below its roofline (BASELINE configurations only, as this library fuses them)
-        own = [r for r in detail if r["key"][0] == "c" and not r["key"].endswith("_reference_rules") and r["key"] != "c2_one_pass"]
-        if own:
-            worst = min(own, key=lambda r: r["roofline"]["frac"])
-            result["worst_config"] = {"name": worst["name"], "frac": worst["roofline"]["frac"], "achieved": worst["roofline"]["achieved"],
-                                      "unit": worst["unit"]}
-    print(json.dumps(result))
+    line, full = final_line(result)
+    if "all_configs" in full and args.detail_out:
+        path = os.path.join(ROOT, args.detail_out)
+        os.makedirs(os.path.dirname(path), exist_ok=True)
+        with open(path, "w") as f:
+            json.dump(full, f, indent=1)
+    print(line)
 
 
 if __name__ == "__main__":
