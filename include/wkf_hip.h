@@ -67,6 +67,10 @@ int wkf_device_props(wkf_device* dev, wkf_props* out);
 int wkf_device_sync(wkf_device* dev);
 /* Return cached free device memory of the buffer pool to the driver. */
 int wkf_device_trim(wkf_device* dev);
+/* Since the device was created: calls of wkf_buffer_alloc, the hipMalloc calls among them (the others were served
+ * by the pool), timers created, and the buffers alive now.  No reference counterpart (wgpu keeps no such count);
+ * lets a caller prove that a call allocated nothing.  Any pointer may be null. */
+int wkf_device_alloc_stats(wkf_device* dev, uint64_t* buffer_allocs, uint64_t* device_mallocs, uint64_t* timers, uint64_t* live_buffers);
 
 /* Replaces create_buffer (zero-initialised by wgpu): src/tensor.rs:334,369,
  * src/element_wise.rs:143, src/reduce.rs:300, src/matmul.rs:167.

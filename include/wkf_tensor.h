@@ -77,11 +77,16 @@ int wkf_device_set_exact_math(wkf_device* dev, int exact);
  * length in one workgroup, src/reduce.rs:340-350, and its composites read such a row once per stage).  Here a row
  * that fits the registers of up to 256 workgroups is computed in ONE launch that reads it once: the workgroups of
  * a row exchange their folded values through memory and wait for each other (all of them are resident: the grid
- * never exceeds four workgroups per compute unit).  The wait is bounded: a lane polls at most `spin_polls` times
- * over the whole kernel (0 = the default, 2^20; the top bit is a test hook that keeps one workgroup per row
- * silent) and then gives up; the next wkf_tensor_as_slice on the device then fails with WKF_ERR_HIP instead of
- * handing out a result.  enabled = 0 goes back to one launch per stage (or one workgroup streaming each row). */
+ * never exceeds what the kernel's registers and the chip's compute units hold).  The wait is bounded: a lane polls
+ * at most `spin_polls` times over the whole kernel (low 31 bits; 0 = the default, 2^20) and then gives up, which
+ * the kernel counts.  wkf_tensor_as_slice / _as_slice_many read that count after their download whenever their own
+ * launches included such a kernel; when it is not zero they compute the tensor a second time with teams off
+ * (one launch per stage, or one workgroup streaming each row) and hand out that result, so a GPU shared with
+ * other work costs time, never a wrong or refused result.  The top bit of `spin_polls` selects a kernel variant
+ * for tests of that path, in which one workgroup per row never publishes its value.  enabled = 0 turns teams off.
+ * wkf_device_row_team_fallbacks: how many read-backs of this device were computed a second time. */
 int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls);
+int wkf_device_row_team_fallbacks(wkf_device* dev, uint64_t* out);
 
 /* Per-kernel GPU timestamps (PerformanceQueries, src/query.rs:50-126: the reference
  * attaches one to every kernel).  On by default; a caller that only wants results can

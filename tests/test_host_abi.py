@@ -614,6 +614,29 @@ def test_reduce_into_plans_without_allocating_and_refuses_the_rest(wkf):
     dev.close()
 
 
+def test_a_timer_outlives_its_device_handle(wkf):
+    # A timer keeps its device alive like a buffer does (its events go back to that device's pool): destroying the
+    # device first and the timer afterwards must find the device still there, and the device goes with the timer.
+    import ctypes
+    lib = wkf.load()
+    lib.wkf_timer_create.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
+    lib.wkf_timer_destroy.argtypes = [ctypes.c_void_p]
+    lib.wkf_timer_destroy.restype = None
+    for _ in range(4):
+        dev = wkf.Device.planner()
+        x = wkf.Tensor.new(dev, np.zeros((8,), dtype=np.float32))
+        stats = dev.alloc_stats()
+        assert stats["live_buffers"] >= 1 and stats["buffer_allocs"] >= 1
+        timers = [ctypes.c_void_p() for _ in range(3)]
+        for t in timers:
+            assert lib.wkf_timer_create(dev._h, ctypes.byref(t)) == 0
+        assert dev.alloc_stats()["timers"] == stats["timers"] + 3
+        dev.close()            # deferred: a buffer and three timers are alive
+        del x                  # the tensor's buffer goes first ...
+        for t in timers:       # ... and the last timer takes the device with it
+            lib.wkf_timer_destroy(t)
+
+
 def _code_object_kernels(path):
     """The kernel records of the AMDGPU metadata note of one code object (ELF note type 32, MessagePack)."""
     import struct
@@ -686,3 +709,38 @@ def test_gemm_kernels_use_no_scratch_memory(tmp_path):
             assert k[".vgpr_spill_count"] == 0 and k[".sgpr_spill_count"] == 0, (k[".name"], k[".vgpr_spill_count"], k[".sgpr_spill_count"])
             assert k[".vgpr_count"] <= 512
     assert checked >= 22, f"only {checked} GEMM kernels were compiled: the shapes above no longer reach the variants"
+
+
+def test_team_row_kernels_fit_four_workgroups_per_compute_unit(tmp_path):
+    # The workgroups of a team wait for each other, so the host sizes the grid for four resident workgroups of 256
+    # lanes per compute unit.  That holds when a kernel needs at most 128 vector registers and no scratch memory;
+    # the launch bounds ask the compiler for exactly that, and its own record in each code object must show it.
+    import glob
+    import subprocess
+    import sys
+    script = (
+        "import sys, numpy as np\n"
+        f"sys.path.insert(0, {os.path.join(ROOT, 'tests')!r})\n"
+        "from helpers import load_package\n"
+        "w = load_package(); dev = w.Device.planner(); T = w.Tensor\n"
+        "for dt, n in ((np.float32, 100003), (np.float32, 131072), (np.float16, 262144), (np.float16, 140002)):\n"
+        "    x = T.new(dev, np.zeros((8, n), dtype=dt)); wt = T.new(dev, np.zeros((n,), dtype=dt))\n"
+        "    for t in (x.softmax_last_dim(), x.layer_norm(wt, 1e-5)):\n"
+        "        t.materialize()\n"
+        "        assert any('teams of' in k.detail for k in t.kernels()), [k.detail for k in t.kernels()]\n"
+        "dev.set_row_teams(True, (1 << 31) | 64)\n"
+        "T.new(dev, np.zeros((8, 100003), dtype=np.float32)).softmax_last_dim().materialize()\n"
+    )
+    env = dict(os.environ, WKF_CACHE_DIR=str(tmp_path))
+    subprocess.run([sys.executable, "-c", script], check=True, env=env, timeout=900)
+    checked = 0
+    for path in glob.glob(os.path.join(str(tmp_path), "*.hsaco")):
+        for k in _code_object_kernels(path):
+            if not k[".name"].startswith("wkf_row"):
+                continue
+            checked += 1
+            assert k[".private_segment_fixed_size"] == 0 and not k[".uses_dynamic_stack"], (k[".name"], k[".private_segment_fixed_size"])
+            assert k[".vgpr_spill_count"] == 0 and k[".sgpr_spill_count"] == 0, (k[".name"], k[".vgpr_spill_count"])
+            assert k[".vgpr_count"] <= 128, (k[".name"], k[".vgpr_count"])
+            assert k[".max_flat_workgroup_size"] == 256
+    assert checked >= 6, f"only {checked} team kernels were compiled"

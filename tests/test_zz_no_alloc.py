@@ -36,10 +36,12 @@ def test_reduce_into_matches_the_allocating_path(gpu, dtype):
         out_shape = tuple(s for d, s in enumerate(shape) if d != axis)
         for attempt in range(2):          # twice: the second call finds the first call's results in the scratch array
             out = w.Tensor.new(gpu, np.full(out_shape, 7.0, dtype=dtype))
-            before = gpu.module_stats()
+            before, held = gpu.module_stats(), gpu.alloc_stats()
             tx.reduce_into(op, axis, out)
             after = gpu.module_stats()
             assert after["compiled"] == before["compiled"] and after["disk_hits"] == before["disk_hits"]
+            # no buffer asked for (neither from the pool nor from hipMalloc), no timer (its events), nothing new alive
+            assert gpu.alloc_stats() == held, (held, gpu.alloc_stats())
             got = out.to_numpy()
             assert got.dtype == want.dtype and got.shape == want.shape
             assert np.array_equal(got, want), f"{shape} axis {axis} {op}: differs from the allocating path"

@@ -37,10 +37,10 @@ EXPORTS = [
     "wkf_device_create", "wkf_device_create_planner", "wkf_device_destroy", "wkf_device_is_planner",
     "wkf_device_props", "wkf_device_sync", "wkf_device_trim", "wkf_buffer_alloc", "wkf_buffer_retain",
     "wkf_buffer_release", "wkf_buffer_refcount", "wkf_buffer_size", "wkf_buffer_ptr", "wkf_buffer_upload",
-    "wkf_buffer_download", "wkf_buffer_copy", "wkf_module_get", "wkf_module_find", "wkf_module_stats", "wkf_launch",
+    "wkf_buffer_download", "wkf_buffer_copy", "wkf_module_get", "wkf_module_find", "wkf_module_stats", "wkf_device_alloc_stats", "wkf_launch",
     "wkf_timer_create", "wkf_timer_destroy", "wkf_timer_begin", "wkf_timer_end", "wkf_timer_elapsed_ns",
     "wkf_last_error",
-    "wkf_device_set_fusion", "wkf_device_get_fusion", "wkf_device_set_exact_math", "wkf_device_set_row_teams", "wkf_device_set_timing", "wkf_tensor_new", "wkf_tensor_clone", "wkf_tensor_free",
+    "wkf_device_set_fusion", "wkf_device_get_fusion", "wkf_device_set_exact_math", "wkf_device_set_row_teams", "wkf_device_row_team_fallbacks", "wkf_device_set_timing", "wkf_tensor_new", "wkf_tensor_clone", "wkf_tensor_free",
     "wkf_tensor_rank", "wkf_tensor_shape", "wkf_tensor_dtype", "wkf_tensor_scalar_op", "wkf_tensor_unary_op",
     "wkf_tensor_cast", "wkf_tensor_binary_op", "wkf_tensor_reduce", "wkf_tensor_reduce_into", "wkf_tensor_mat_mul", "wkf_tensor_slice",
     "wkf_tensor_transpose", "wkf_tensor_broadcast", "wkf_tensor_narrow", "wkf_tensor_resize",
@@ -150,7 +150,9 @@ def load():
     lib.wkf_device_set_exact_math.argtypes = [c_void_p, c_int]
     lib.wkf_device_set_timing.argtypes = [c_void_p, c_int]
     lib.wkf_device_set_row_teams.argtypes = [c_void_p, c_int, ctypes.c_uint32]
+    lib.wkf_device_row_team_fallbacks.argtypes = [c_void_p, POINTER(c_uint64)]
     lib.wkf_module_stats.argtypes = [c_void_p, POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]
+    lib.wkf_device_alloc_stats.argtypes = [c_void_p, POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]
     lib.wkf_buffer_alloc.argtypes = [c_void_p, c_size_t, c_int, POINTER(c_void_p)]
     lib.wkf_buffer_release.argtypes = [c_void_p]
     lib.wkf_buffer_release.restype = None
@@ -285,10 +287,21 @@ class Device:
         wkf_device_set_row_teams.  spin_polls = 0 keeps the default bound of the wait."""
         _check(self._lib.wkf_device_set_row_teams(self._h, 1 if enabled else 0, int(spin_polls)))
 
+    def row_team_fallbacks(self):
+        """Read-backs that were computed a second time, without teams, because a team kernel gave up waiting."""
+        n = c_uint64()
+        _check(self._lib.wkf_device_row_team_fallbacks(self._h, byref(n)))
+        return n.value
+
     def module_stats(self):
         a, b, c = c_uint64(), c_uint64(), c_uint64()
         _check(self._lib.wkf_module_stats(self._h, byref(a), byref(b), byref(c)))
         return {"compiled": a.value, "disk_hits": b.value, "mem_hits": c.value}
+
+    def alloc_stats(self):
+        a, b, c, d = c_uint64(), c_uint64(), c_uint64(), c_uint64()
+        _check(self._lib.wkf_device_alloc_stats(self._h, byref(a), byref(b), byref(c), byref(d)))
+        return {"buffer_allocs": a.value, "device_mallocs": b.value, "timers": c.value, "live_buffers": d.value}
 
     def close(self):
         if self._h:

@@ -958,6 +958,7 @@ std::string row_signature(const RowSpec& s) {
   if (s.online_max_sum) o << "|online";
   if (s.split) o << "|split" << s.split_phase;
   if (s.team) o << "|team";
+  if (s.team && s.team_mute) o << "|mute";
   return o.str();
 }
 
@@ -1060,8 +1061,9 @@ std::string row_source(const RowSpec& s) {
     o << "  const u32 teams = gridDim.x / a.parts;\n";
     o << "  u64* const slots = (u64*)a.p[" << K + 1 << "];\n";
     o << "  u64* const gave_up = (u64*)a.p[" << K + 2 << "];\n";
-    o << "  u32 polls_left = a.spin & 0x7fffffffu;\n";
-    o << "  const bool mute = (a.spin >> 31) != 0u && part == 0u;  // host-side test of the give-up path: part 0 never writes its slots\n";
+    o << "  u32 polls_left = a.spin;\n";
+    // a variant of its own for the host-side test of the give-up path: part 0 never writes its slots
+    const std::string may_put = s.team_mute ? " && part != 0u" : "";
     for (int k = 0; k < S; k++) {
       const bool online = s.online_max_sum && k < 2;
       o << "  auto fold" << k << " = [](float v, float a) { return " << fold_text(online ? (k == 0 ? ReduceOp::Max : ReduceOp::Sum) : s.stages[k].rop)
@@ -1182,7 +1184,7 @@ std::string row_source(const RowSpec& s) {
         own_fold(1, "    ");
         o << "  }\n";
         o << "  if (talk_wave) {\n";
-        o << "    if (t == " << XL << "u && !mute) {\n      wkf_team_put(" << slot(0, "part") << ", acc0);\n      wkf_team_put(" << slot(1, "part") << ", acc1);\n    }\n";
+        o << "    if (t == " << XL << "u" << may_put << ") {\n      wkf_team_put(" << slot(0, "part") << ", acc0);\n      wkf_team_put(" << slot(1, "part") << ", acc1);\n    }\n";
         o << "    float row_max = " << seed_text(ReduceOp::Max) << ", row_sum = 0.0f;\n";
         o << "    for (u32 p = t - " << XL << "u; p < a.parts; p += 64u) {\n";
         o << "      float part_max, part_sum;\n";
@@ -1207,7 +1209,7 @@ std::string row_source(const RowSpec& s) {
       o << "  float acc" << k << " = " << seed_text(s.stages[k].rop) << ";\n";
       own_fold(k, "  ");
       o << "  if (talk_wave) {\n";
-      o << "    if (t == " << XL << "u && !mute) wkf_team_put(" << slot(k, "part") << ", acc" << k << ");\n";
+      o << "    if (t == " << XL << "u" << may_put << ") wkf_team_put(" << slot(k, "part") << ", acc" << k << ");\n";
       o << "    float v = " << seed_text(s.stages[k].rop) << ";\n";
       o << "    for (u32 p = t - " << XL << "u; p < a.parts; p += 64u) {\n";
       o << "      float pa, pb;\n";

@@ -167,6 +167,7 @@ struct RowSpec {
   // resident: the grid is teams * parts blocks with at most four blocks per compute unit, and a team walks rows
   // team, team + teams, ...  The last pointer argument counts the lanes that gave up waiting (see `spin`).
   bool team = false;
+  bool team_mute = false;               // a variant for host-side tests of the give-up path: part 0 of every row never writes its slots
   std::vector<ReduceOperandSpec> in;    // axis_stride 1 (row in registers) or 0 (one scalar per row)
   std::vector<RowStage> stages;
   Program final;                        // same operand numbering as a stage's pre
@@ -183,8 +184,7 @@ struct RowArgs {
   uint32_t nrows;
   uint32_t nvec = 0;                              // ragged and streamed kernels only: vectors per row
   uint32_t parts = 0, chunk = 0;                  // split kernels: parts per row, vectors per part; team kernels: parts
-  uint32_t spin = 0;                              // team kernels: polls a lane may spend waiting over the whole kernel (low 31 bits);
-                                                  // top bit: part 0 never writes its slots (test of the give-up path)
+  uint32_t spin = 0;                              // team kernels: polls a lane may spend waiting over the whole kernel
   std::vector<uint32_t> oshape;
   std::vector<uint32_t> offsets;                  // per operand incl. outputs
   std::vector<std::vector<uint32_t>> ostrides;    // per operand incl. outputs, per outer dim

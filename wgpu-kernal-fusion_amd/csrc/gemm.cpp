@@ -255,7 +255,13 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     size_t S = (want + gridx * batch - 1) / (gridx * batch);
     S = std::min(S, std::max<size_t>(1, K * dtype_size(a.dtype) / (8 * M)));  // partial sums stay under half of W's bytes
     S = std::min(S, std::max<size_t>(1, K / (2 * kblock)));
-    if (valu) S = std::max(S, (K + 2047) / 2048);  // the LDS holds at most 2048 elements of each row of A
+    if (valu) {
+      // the block's slice of A lives in static LDS, [M][chunk_max] with chunk_max a power of two: at most 2048
+      // elements of each row and at most 64 KiB in all, so that several blocks share a compute unit
+      size_t lim = 2048;
+      while (lim > 256 && M * lim * dtype_size(a.dtype) > 65536) lim /= 2;
+      S = std::max(S, (K + lim - 1) / lim);
+    }
     size_t chunk = (K + S - 1) / S;
     chunk = (chunk + kblock - 1) / kblock * kblock;
     S = (K + chunk - 1) / chunk;

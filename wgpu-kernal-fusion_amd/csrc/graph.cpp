@@ -234,6 +234,7 @@ namespace {
 struct TeamWord {
   BufRef buf;
   bool pending = false;
+  uint64_t fallbacks = 0;
 };
 std::mutex g_team_mu;
 std::unordered_map<wkf_device*, TeamWord> g_team;
@@ -260,28 +261,43 @@ void* team_word(wkf_device* dev) {
   w.pending = true;
   return wkf_buffer_ptr(w.buf.get());
 }
+// the word of `dev` when team kernels ran since it was last read (and marks it read), else nothing
+BufRef team_take_pending(wkf_device* dev) {
+  std::lock_guard<std::mutex> lock(g_team_mu);
+  auto it = g_team.find(dev);
+  if (it == g_team.end() || !it->second.pending) return BufRef();
+  it->second.pending = false;
+  return it->second.buf;
+}
 }  // namespace
 
-void team_check(wkf_device* dev) {
-  BufRef buf;
-  {
-    std::lock_guard<std::mutex> lock(g_team_mu);
-    auto it = g_team.find(dev);
-    if (it == g_team.end() || !it->second.pending) return;
-    it->second.pending = false;
-    buf = it->second.buf;
-  }
-  if (wkf_device_is_planner(dev)) return;
-  unsigned long long n = 0;
-  check(wkf_buffer_download(buf.get(), 0, &n, sizeof n));
-  if (n == 0) return;
-  const unsigned long long zero = 0;
+void team_begin(wkf_device* dev) {
+  BufRef buf = team_take_pending(dev);
+  if (!buf || wkf_device_is_planner(dev)) return;
+  const unsigned long long zero = 0;  // in stream order: after the launches that may still count, before the ones to come
   check(wkf_buffer_upload(buf.get(), 0, &zero, sizeof zero));
-  throw Error(WKF_ERR_HIP, "a row kernel whose blocks wait for each other gave up waiting (" + std::to_string(n) +
-                               " lanes): results computed since the last read-back are not valid");
 }
 
-TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero) {
+bool team_gave_up(wkf_device* dev) {
+  BufRef buf = team_take_pending(dev);
+  if (!buf || wkf_device_is_planner(dev)) return false;
+  unsigned long long n = 0;
+  check(wkf_buffer_download(buf.get(), 0, &n, sizeof n));
+  if (n == 0) return false;
+  const unsigned long long zero = 0;
+  check(wkf_buffer_upload(buf.get(), 0, &zero, sizeof zero));
+  std::lock_guard<std::mutex> lock(g_team_mu);
+  g_team[dev].fallbacks++;
+  return true;
+}
+
+uint64_t team_fallbacks(wkf_device* dev) {
+  std::lock_guard<std::mutex> lock(g_team_mu);
+  auto it = g_team.find(dev);
+  return it == g_team.end() ? 0 : it->second.fallbacks;
+}
+
+TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero, bool result) {
   TensorData td;
   td.device = dev_;
   td.layout = Layout::contiguous(shape);
@@ -292,7 +308,11 @@ TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero
   if (noalloc_) {
     // nothing is allocated: the result is the caller's tensor, a temporary is the device's static scratch array
     if (zero) throw Error(WKF_ERR_UNSUPPORTED, "allocation-free call: the graph needs a zero-filled buffer");
-    if (!noalloc_->out_taken && shape == noalloc_->out.layout.shape && dt == noalloc_->out.dtype) {
+    if (result) {
+      // the launch that finishes the reduction writes the caller's tensor: bound to it by role, not by a shape that
+      // a temporary might share
+      if (noalloc_->out_taken || shape != noalloc_->out.layout.shape || dt != noalloc_->out.dtype)
+        throw Error(WKF_ERR_UNSUPPORTED, "allocation-free call: the result does not fit the output tensor");
       noalloc_->out_taken = true;
       return noalloc_->out;
     }
@@ -820,6 +840,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   spec.ragged = ragged;
   spec.streamed = streamed;
   spec.team = team;
+  spec.team_mute = team && st_.row_team_test_mute;
   spec.stages = rb.stages;
   if ((streamed || team) && rb.stages.size() >= 2) {
     // softmax's pair of stages, max(x) then sum(exp(x - max)), is folded in one pass over a streamed row
@@ -878,6 +899,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
     args.ptrs.push_back(team_word(dev_));
     args.parts = to_u32(parts, "parts");
     args.spin = st_.row_team_spin;
+    team_launched_ = true;
     std::string sig = row_signature(spec);
     wkf_kernel* k = kernel(sig, [&] { return row_source(spec); });
     LaunchRecord r;
@@ -1361,7 +1383,8 @@ TensorData Resolver::launch_reduce(const ReduceJob& job) {
   std::vector<size_t> out_shape;
   for (size_t d = 0; d < shape.size(); d++)
     if (d != axis) out_shape.push_back(shape[d]);
-  TensorData out = alloc(out_shape, out_dt, false);
+  // (raw partial sums are a temporary; anything else a reduce launch stores is the value of its reduce node)
+  TensorData out = alloc(out_shape, out_dt, false, !job.raw);
   const size_t nrows = out.layout.numel();
   const size_t n = shape[axis];
   if (nrows == 0) return out;

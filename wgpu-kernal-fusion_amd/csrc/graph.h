@@ -45,7 +45,8 @@ struct Settings {
   int reduce_unroll = 0;          // loads in flight per lane in row reduces; 0 = chosen (WKF_REDUCE_UNROLL overrides)
   bool row_split = true;             // rows too long for a block's registers and too few to stream with a block each: one launch per stage over parts of rows (WKF_ROW_SPLIT=0: fold each reduction across the grid instead)
   bool row_team = true;              // rows too long for a block's registers that fit those of up to 256 blocks: one launch, the row read once, the blocks of a row exchange their folds and wait for each other (WKF_ROW_TEAM=0 turns it off)
-  uint32_t row_team_spin = 1u << 20; // polls a lane of such a kernel may spend waiting before it gives up (the result is then refused at read-back); top bit: part 0 stays silent (tests)
+  uint32_t row_team_spin = 1u << 20; // polls a lane of such a kernel may spend waiting before it gives up (the read-back then computes the tensor again without teams)
+  bool row_team_test_mute = false;   // tests of that path: a kernel variant in which part 0 of every row stays silent
   size_t row_stream_min_rows = 256;  // fewest rows for the one-launch kernel that streams rows longer than a block's registers (WKF_ROW_STREAM_MIN_ROWS)
 };
 
@@ -57,10 +58,15 @@ struct Space {
   std::vector<std::vector<size_t>> strides;  // [operand][dim]
 };
 
-// Team row kernels count the lanes that gave up waiting for another block in one word per device.  Called after a
-// download has synchronised the stream: throws when the count is not zero (and clears it), so that no result of
-// such a kernel, or of anything computed from it, is handed out unnoticed.
-void team_check(wkf_device* dev);
+// Team row kernels count the lanes that gave up waiting for another block in one word per device.
+// team_begin: before a read-back starts its launches; clears a count left by launches nobody read back.
+// team_gave_up: after the read-back's download has synchronised the stream and only when its own launches
+// included a team kernel; true (and the count cleared) when a lane gave up, so that the caller computes the
+// tensor again without teams instead of handing that result out.
+void team_begin(wkf_device* dev);
+bool team_gave_up(wkf_device* dev);
+// read-backs that were computed a second time for that reason, per device (tests)
+uint64_t team_fallbacks(wkf_device* dev);
 
 class Resolver {
  public:
@@ -77,6 +83,8 @@ class Resolver {
     bool out_taken = false, scratch_taken = false;
   };
   void set_noalloc(NoAlloc* na) { noalloc_ = na; }
+  // whether any launch of this resolver was a team row kernel (whose result needs team_gave_up before it leaves)
+  bool team_launched() const { return team_launched_; }
 
  private:
   TensorData resolve(const NodeP& n);
@@ -142,13 +150,15 @@ class Resolver {
   void launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place,
                   const std::vector<Program>& more_prog = {}, const std::vector<TensorData>& more_out = {});
   void launch_map_tiled(MapSpec& spec, const Space& sp, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
-  TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero);
+  // `result`: the buffer receives the value of a reduce node (allocation-free mode: the caller's output tensor)
+  TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero, bool result = false);
   TensorData make_contiguous(const TensorData& td);
   void record(LaunchRecord&& r, wkf_kernel* k, const std::vector<unsigned char>& args);
   wkf_kernel* kernel(const std::string& sig, const std::function<std::string()>& make_body);
 
   wkf_device* dev_;
   NoAlloc* noalloc_ = nullptr;
+  bool team_launched_ = false;
   Settings st_;
   std::vector<LaunchRecord>* log_;
   std::set<const Node*> shared_;

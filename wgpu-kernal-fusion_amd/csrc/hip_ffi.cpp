@@ -121,7 +121,10 @@ struct wkf_device {
   wkf_props props{};
   // buffers handed out and not yet released; a destroy with some still alive is deferred to the last release
   size_t live_buffers = 0;
+  size_t live_timers = 0;  // timers keep the device the same way (their events go back to this device's pool)
   bool closing = false;
+  // since the device was created: calls of wkf_buffer_alloc, of hipMalloc among them, and of wkf_timer_create
+  uint64_t n_buffer_allocs = 0, n_device_mallocs = 0, n_timers = 0;
   // timed launches take their events inside the dispatch (WKF_TIMER_EVENTS=1: two recorded events around it instead)
   bool timer_in_dispatch = [] { const char* e = getenv("WKF_TIMER_EVENTS"); return !(e && atoi(e) != 0); }();
   // events of destroyed timers, handed out again by wkf_timer_create: a timed launch costs two event
@@ -293,7 +296,7 @@ void wkf_device_destroy(wkf_device* dev) {
     // then lives on until the last of them is released, so that a late wkf_buffer_release / wkf_tensor_free
     // never touches freed memory.
     std::lock_guard<std::recursive_mutex> lock(dev->mu);
-    if (dev->live_buffers > 0) {
+    if (dev->live_buffers > 0 || dev->live_timers > 0) {
       dev->closing = true;
       return;
     }
@@ -323,6 +326,16 @@ int wkf_device_props(wkf_device* dev, wkf_props* out) {
   return WKF_OK;
 }
 
+int wkf_device_alloc_stats(wkf_device* dev, uint64_t* buffer_allocs, uint64_t* device_mallocs, uint64_t* timers, uint64_t* live_buffers) {
+  if (!dev) return fail(WKF_ERR_INVALID_ARG, "wkf_device_alloc_stats: null device");
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  if (buffer_allocs) *buffer_allocs = dev->n_buffer_allocs;
+  if (device_mallocs) *device_mallocs = dev->n_device_mallocs;
+  if (timers) *timers = dev->n_timers;
+  if (live_buffers) *live_buffers = dev->live_buffers;
+  return WKF_OK;
+}
+
 int wkf_device_sync(wkf_device* dev) {
   if (!dev) return fail(WKF_ERR_INVALID_ARG, "wkf_device_sync: null device");
   if (dev->planner) return WKF_OK;
@@ -334,6 +347,7 @@ int wkf_device_sync(wkf_device* dev) {
 int wkf_buffer_alloc(wkf_device* dev, size_t bytes, int zero_fill, wkf_buffer** out) {
   if (!dev || !out) return fail(WKF_ERR_INVALID_ARG, "wkf_buffer_alloc: null argument");
   std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  dev->n_buffer_allocs++;
   size_t cap = pool_bucket(bytes);
   void* ptr = nullptr;
   auto it = dev->pool.find(cap);
@@ -346,6 +360,7 @@ int wkf_buffer_alloc(wkf_device* dev, size_t bytes, int zero_fill, wkf_buffer** 
     if (!ptr) return fail(WKF_ERR_OOM, "wkf_buffer_alloc: host allocation failed");
   } else {
     WKF_HIP_CHECK(hipSetDevice(dev->ordinal));
+    dev->n_device_mallocs++;
     hipError_t e = hipMalloc(&ptr, cap);
     if (e == hipErrorOutOfMemory) {
       // Give cached blocks back to the driver and retry once.
@@ -385,7 +400,7 @@ void wkf_buffer_release(wkf_buffer* buf) {
   bool last = false;
   {
     std::lock_guard<std::recursive_mutex> lock(dev->mu);
-    last = --dev->live_buffers == 0 && dev->closing;
+    last = --dev->live_buffers == 0 && dev->live_timers == 0 && dev->closing;
     // Work already queued on the single stream finishes before any later user of
     // this block starts, so the block can be handed out again without a sync.
     if (dev->pool_bytes + buf->capacity <= dev->pool_limit) {
@@ -616,8 +631,9 @@ int wkf_timer_create(wkf_device* dev, wkf_timer** out) {
   if (!dev || !out) return fail(WKF_ERR_INVALID_ARG, "wkf_timer_create: null argument");
   wkf_timer* t = new wkf_timer();
   t->dev = dev;
+  std::lock_guard<std::recursive_mutex> lock(dev->mu);
+  dev->n_timers++;
   if (!dev->planner) {
-    std::lock_guard<std::recursive_mutex> lock(dev->mu);
     hipEvent_t* slot[2] = {&t->begin, &t->end};
     for (hipEvent_t* e : slot) {
       if (!dev->free_events.empty()) {
@@ -630,18 +646,24 @@ int wkf_timer_create(wkf_device* dev, wkf_timer** out) {
       }
     }
   }
+  dev->live_timers++;
   *out = t;
   return WKF_OK;
 }
 
 void wkf_timer_destroy(wkf_timer* t) {
   if (!t) return;
+  wkf_device* dev = t->dev;
+  bool last = false;
   {
-    std::lock_guard<std::recursive_mutex> lock(t->dev->mu);
-    if (t->begin) t->dev->free_events.push_back(t->begin);
-    if (t->end) t->dev->free_events.push_back(t->end);
+    std::lock_guard<std::recursive_mutex> lock(dev->mu);
+    if (t->begin) dev->free_events.push_back(t->begin);
+    if (t->end) dev->free_events.push_back(t->end);
+    // a timer destroyed after wkf_device_destroy: the device was kept for it, like for a live buffer
+    last = --dev->live_timers == 0 && dev->live_buffers == 0 && dev->closing;
   }
   delete t;
+  if (last) destroy_now(dev);
 }
 
 int wkf_timer_begin(wkf_timer* t) {

@@ -468,7 +468,16 @@ int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls) 
     settings_for(dev);
     std::lock_guard<std::mutex> lock(g_settings_mu);
     g_settings[dev].row_team = enabled != 0;
-    g_settings[dev].row_team_spin = spin_polls == 0 ? Settings().row_team_spin : spin_polls;
+    g_settings[dev].row_team_spin = (spin_polls & 0x7fffffffu) == 0 ? Settings().row_team_spin : (spin_polls & 0x7fffffffu);
+    g_settings[dev].row_team_test_mute = (spin_polls >> 31) != 0;
+  });
+}
+
+int wkf_device_row_team_fallbacks(wkf_device* dev, uint64_t* out) {
+  return guarded([&] {
+    need(dev, "wkf_device_row_team_fallbacks");
+    need(out, "wkf_device_row_team_fallbacks");
+    *out = team_fallbacks(dev);
   });
 }
 
@@ -777,12 +786,24 @@ int wkf_tensor_arange(wkf_device* dev, int dtype, float start, float end, float 
   });
 }
 
-static TensorData materialize(wkf_tensor* t) {
+// `st`: the settings to resolve under (null: the device's); `*team` tells whether a team row kernel was launched
+static TensorData materialize(wkf_tensor* t, const Settings* st = nullptr, bool* team = nullptr) {
   for (LaunchRecord& r : t->launches)
     if (r.timer) wkf_timer_destroy(r.timer);
   t->launches.clear();
-  Resolver res(t->dev, settings_for(t->dev), &t->launches);
-  return res.resolve_root(t->node);
+  Resolver res(t->dev, st ? *st : settings_for(t->dev), &t->launches);
+  TensorData td = res.resolve_root(t->node);
+  if (team) *team = res.team_launched();
+  return td;
+}
+
+// The settings of `dev` with team row kernels off: what a read-back resolves under, a second time, when a team
+// kernel of its first pass gave up waiting.  The graph is still lazy and its leaves are never written in place,
+// so the second pass computes the same tensor from the same inputs, one launch per stage or a block per row.
+static Settings without_teams(wkf_device* dev) {
+  Settings st = settings_for(dev);
+  st.row_team = false;
+  return st;
 }
 
 int wkf_tensor_materialize(wkf_tensor* t) {
@@ -792,7 +813,7 @@ int wkf_tensor_materialize(wkf_tensor* t) {
   });
 }
 
-static std::vector<TensorData> materialize_many(wkf_tensor** ts, int n, const char* who) {
+static std::vector<TensorData> materialize_many(wkf_tensor** ts, int n, const char* who, const Settings* st = nullptr, bool* team = nullptr) {
   need(ts, who);
   if (n <= 0) invalid(std::string(who) + ": no tensors");
   std::vector<NodeP> roots;
@@ -805,8 +826,10 @@ static std::vector<TensorData> materialize_many(wkf_tensor** ts, int n, const ch
     roots.push_back(ts[i]->node);
   }
   // every launch of the joint pass is recorded on the first tensor
-  Resolver res(ts[0]->dev, settings_for(ts[0]->dev), &ts[0]->launches);
-  return res.resolve_roots(roots);
+  Resolver res(ts[0]->dev, st ? *st : settings_for(ts[0]->dev), &ts[0]->launches);
+  std::vector<TensorData> tds = res.resolve_roots(roots);
+  if (team) *team = res.team_launched();
+  return tds;
 }
 
 int wkf_tensor_materialize_many(wkf_tensor** ts, int n) {
@@ -896,21 +919,32 @@ std::string graph_dot(const NodeP& root) {
 }  // namespace
 }  // extern "C++"
 
+static std::unique_ptr<wkf_slice> download_slice(const TensorData& td) {
+  std::unique_ptr<wkf_slice> s(new wkf_slice());
+  s->layout = td.layout;
+  s->dtype = td.dtype;
+  s->bytes.resize(wkf_buffer_size(td.buffer.get()));
+  int rc = wkf_buffer_download(td.buffer.get(), 0, s->bytes.data(), s->bytes.size());
+  if (rc != WKF_OK) throw Error(rc, wkf_last_error());
+  return s;
+}
+
 int wkf_tensor_as_slice_many(wkf_tensor** ts, int n, wkf_slice** out) {
   return guarded([&] {
     need(out, "wkf_tensor_as_slice_many");
-    std::vector<TensorData> tds = materialize_many(ts, n, "wkf_tensor_as_slice_many");
+    need(ts, "wkf_tensor_as_slice_many");
+    if (n > 0 && ts[0]) team_begin(ts[0]->dev);
     std::vector<std::unique_ptr<wkf_slice>> slices;
-    for (const TensorData& td : tds) {
-      std::unique_ptr<wkf_slice> s(new wkf_slice());
-      s->layout = td.layout;
-      s->dtype = td.dtype;
-      s->bytes.resize(wkf_buffer_size(td.buffer.get()));
-      int rc = wkf_buffer_download(td.buffer.get(), 0, s->bytes.data(), s->bytes.size());
-      if (rc != WKF_OK) throw Error(rc, wkf_last_error());
-      slices.push_back(std::move(s));
+    bool team = false;
+    std::vector<TensorData> tds = materialize_many(ts, n, "wkf_tensor_as_slice_many", nullptr, &team);
+    for (const TensorData& td : tds) slices.push_back(download_slice(td));
+    if (team && team_gave_up(ts[0]->dev)) {  // every tensor of the call is on that device
+      slices.clear();
+      tds.clear();
+      const Settings st = without_teams(ts[0]->dev);
+      tds = materialize_many(ts, n, "wkf_tensor_as_slice_many", &st);
+      for (const TensorData& td : tds) slices.push_back(download_slice(td));
     }
-    if (n > 0) team_check(tds[0].device);
     for (int i = 0; i < n; i++) out[i] = slices[size_t(i)].release();
   });
 }
@@ -928,14 +962,17 @@ int wkf_tensor_as_slice(wkf_tensor* t, wkf_slice** out) {
   return guarded([&] {
     need(t, "wkf_tensor_as_slice");
     need(out, "wkf_tensor_as_slice");
-    TensorData td = materialize(t);
-    std::unique_ptr<wkf_slice> s(new wkf_slice());
-    s->layout = td.layout;
-    s->dtype = td.dtype;
-    s->bytes.resize(wkf_buffer_size(td.buffer.get()));
-    int rc = wkf_buffer_download(td.buffer.get(), 0, s->bytes.data(), s->bytes.size());
-    if (rc != WKF_OK) throw Error(rc, wkf_last_error());
-    team_check(td.device);
+    team_begin(t->dev);
+    bool team = false;
+    TensorData td = materialize(t, nullptr, &team);
+    std::unique_ptr<wkf_slice> s = download_slice(td);
+    if (team && team_gave_up(t->dev)) {
+      s.reset();
+      td = TensorData();
+      const Settings st = without_teams(t->dev);
+      td = materialize(t, &st);
+      s = download_slice(td);
+    }
     *out = s.release();
   });
 }
