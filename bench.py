@@ -621,6 +621,93 @@ def _raw_timed(lib, dev, fn, reps, warm):
     return ns.value / reps / 1e3
 
 
+def _smi_sample():
+    """One reading of the GPU's power and clocks from rocm-smi (a child process), or the error it gave."""
+    try:
+        r = subprocess.run(["rocm-smi", "--showpower", "--showmaxpower", "--showclocks", "--json"], capture_output=True, text=True, timeout=10)
+        card = next(iter(json.loads(r.stdout).values()))
+    except Exception as e:  # no rocm-smi, no permission, no JSON: the row then says so
+        return {"error": repr(e)[:200]}
+    keep = {}
+    for k, v in card.items():
+        lk = k.lower()
+        if "power" in lk or "sclk" in lk or "mclk" in lk or "fclk" in lk:
+            keep[k] = v
+    return keep
+
+
+def power_rows(w, dev, seeded, seconds):
+    """`--yardstick power`: what the chip draws and clocks at while it runs (a) the library's f16 4096^3 product,
+    (b) the MFMA-only loop on the same operands, (c) the MFMA-only loop on zeros, (d) nothing.  Every phase enqueues
+    its kernel back to back for `seconds` while a thread reads rocm-smi; the rows carry every reading and the rate."""
+    import struct
+    import threading
+    from ctypes import byref, c_uint32, c_void_p
+    lib = w.load()
+    T = w.Tensor
+    ha = seeded(5, 0, (4096, 4096), "normal", dtype=np.float16, std=0.02)
+    hb = seeded(5, 1, (4096, 4096), "normal", dtype=np.float16, std=0.02)
+    a16, b16 = T.new(dev, ha), T.new(dev, hb)
+    prod = a16.mat_mul(b16)
+    k = c_void_p()
+    assert lib.wkf_module_get(dev._h, b"yardstick|mfma_only|32x32x16", MFMA_ONLY_SRC.encode(), b"wkf_mfma_only", byref(k)) == 0, lib.wkf_last_error()
+
+    def raw(host):
+        buf = c_void_p()
+        assert lib.wkf_buffer_alloc(dev._h, host.nbytes, 1, byref(buf)) == 0
+        assert lib.wkf_buffer_upload(buf, 0, host.ctypes.data_as(c_void_p), host.nbytes) == 0
+        return buf
+
+    ba, bb, bz, bc = raw(ha), raw(hb), raw(np.zeros((4096, 4096), np.float16)), raw(np.zeros((256, 256), np.float16))
+    grid, block = (c_uint32 * 3)(256, 1, 1), (c_uint32 * 3)(256, 1, 1)
+
+    def mfma_only(x, y):
+        args = struct.pack("PPPIIII", lib.wkf_buffer_ptr(x), lib.wkf_buffer_ptr(y), lib.wkf_buffer_ptr(bc), 4096, 4096, 4096, 0)
+        return lambda: lib.wkf_launch(dev._h, k, grid, block, 0, args, len(args), None)
+
+    dev.set_timing(False)
+    phases = [("library GEMM f16 4096^3, config-5 operands", lambda: prod.materialize()),
+              ("MFMA only, config-5 operands", mfma_only(ba, bb)),
+              ("MFMA only, zeros", mfma_only(bz, bz)),
+              ("idle", None)]
+    rows = []
+    for name, fn in phases:
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            time.sleep(0.5)  # let the clocks settle under the load first
+            while not stop.is_set():
+                s = _smi_sample()
+                s["t"] = round(time.perf_counter() - t0, 2)
+                samples.append(s)
+                time.sleep(0.2)
+
+        t0 = time.perf_counter()
+        th = threading.Thread(target=sampler)
+        th.start()
+        launches = 0
+        if fn is None:
+            time.sleep(seconds)
+        else:
+            while time.perf_counter() - t0 < seconds:
+                for _ in range(200):
+                    fn()
+                dev.sync()
+                launches += 200
+        elapsed = time.perf_counter() - t0
+        stop.set()
+        th.join()
+        row = {"phase": name, "seconds": round(elapsed, 2), "launches": launches, "smi": samples}
+        if launches:
+            row["us_per_launch_wall"] = round(elapsed / launches * 1e6, 2)
+            row["TFLOP/s"] = round(2 * 4096 ** 3 * launches / elapsed * 1e-12, 1)
+        rows.append(row)
+    dev.set_timing(True)
+    for bf in (ba, bb, bz, bc):
+        lib.wkf_buffer_release(bf)
+    return rows
+
+
 def yardsticks(w, dev, seeded, which, launches):
     """`--yardstick mfma|stream`: kernels that are not part of the library, launched through its level-0 ABI, which
     bound what the library's kernels can reach on this machine: the matrix cores alone on the benchmark's operand
@@ -703,8 +790,10 @@ def yardsticks(w, dev, seeded, which, launches):
         for name in ("copy", "read-only", "write-only", "two reads + one write"):
             best = max((r for r in rows if r["what"].startswith(name)), key=lambda r: r["GB/s"])
             out["best_" + name.replace("-", "_").replace(" + ", "_").replace(" ", "_")] = best
+    elif which == "power":
+        out["phases"] = power_rows(w, dev, seeded, max(2.0, launches / 10.0))
     else:
-        sys.exit("bench.py --yardstick: mfma or stream")
+        sys.exit("bench.py --yardstick: mfma, stream or power")
     print(json.dumps(out))
 
 
@@ -756,7 +845,8 @@ def main():
     ap.add_argument("--warm-ms", type=float, default=300.0, help="--profile: milliseconds of untimed steps before the timed ones")
     ap.add_argument("--detail-out", default="gpurun_out/bench_detail.json",
                     help="file (relative to this one) that receives the full record with every row; empty: none")
-    ap.add_argument("--yardstick", default="", help="mfma | stream: bounds of the machine measured with kernels outside the library")
+    ap.add_argument("--yardstick", default="", help="mfma | stream: bounds of the machine measured with kernels outside the library; "
+                                                    "power: rocm-smi readings while the f16 product and the MFMA-only loops run (--launches/10 seconds each)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU (every kernel, no collectives); --gpus must be 1.")

@@ -459,7 +459,9 @@ def test_mat_mul_kernel_choice(wkf, planner):
         assert _kinds(t) == ["gemm"]
         return t.kernels()[0].detail
 
-    assert detail(4096, 4096, 128, np.float16).endswith("mfma 256x256 tiles")
+    # full f16 tiles: the operands go from memory straight into the LDS (whole tiles and a last round in half tiles)
+    assert detail(4096, 4096, 192, np.float16).endswith("mfma 256x256 tiles, operands loaded straight into the LDS")
+    assert detail(4096, 4352, 192, np.float16).endswith("operands loaded straight into the LDS, last round: 16 tiles as 32 halves of 128 rows")
     assert detail(512, 256, 96, np.float32).endswith("mfma 256x256 tiles")
     # not a multiple of the tile but every row 16-byte aligned: the same MFMA kernel with edge handling
     assert detail(4000, 4000, 72, np.float16).endswith("mfma 256x256 tiles edge")
@@ -470,7 +472,7 @@ def test_mat_mul_kernel_choice(wkf, planner):
     # f16 products whose large tiles would fill at most half of the chip take 128 x 128 tiles, two workgroups per compute unit
     assert detail(512, 256, 128, np.float16).endswith("mfma 128x128 tiles")
     assert detail(300, 264, 72, np.float16).endswith("mfma 128x128 tiles")
-    assert detail(1024, 11008, 512, np.float16).endswith("mfma 256x256 tiles")
+    assert detail(1024, 11008, 512, np.float16).endswith("mfma 256x256 tiles, operands loaded straight into the LDS")
     # unaligned rows or tiny problems: the generic kernel
     assert detail(300, 262, 72, np.float16).endswith("generic")
     assert detail(3, 7, 5, np.float32).endswith("generic")
@@ -491,6 +493,9 @@ def test_mat_mul_kernel_choice(wkf, planner):
     w = _x(wkf, planner, (512, 256), np.float16, seed=2)
     t = _x(wkf, planner, (256, 256), np.float16).mat_mul(w.transpose(0, 1))
     assert _kinds(t) == ["gemm"] and t.kernels()[0].detail.endswith("B^T") and "|bt" in t.kernels()[0].signature
+    big_w = _x(wkf, planner, (4096, 256), np.float16, seed=2)
+    t = _x(wkf, planner, (4096, 256), np.float16).mat_mul(big_w.transpose(0, 1))
+    assert _kinds(t) == ["gemm"] and "B^T" in t.kernels()[0].detail and t.kernels()[0].signature.endswith("|bt|direct to LDS")
     # ... and with a handful of rows W is streamed once through MFMA operands (decode)
     t = _x(wkf, planner, (2, 256), np.float16).mat_mul(w.transpose(0, 1))
     assert _kinds(t)[0] == "gemm" and "skinny B^T" in t.kernels()[0].detail and t.shape() == (2, 512)

@@ -38,6 +38,9 @@ const char* const kGemmSkinnyTr =
 const char* const kGemmF16T128 =
 #include "kernels/gemm_f16_t128.hip.inc"
     ;
+const char* const kGemmF16Dma =
+#include "kernels/gemm_f16_dma.hip.inc"
+    ;
 const char* const kGemmF16Tail =
 #include "kernels/gemm_f16_tail.hip.inc"
     ;
@@ -475,7 +478,11 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // half as long (kernels/gemm_f16_tail.hip.inc, kernels/gemm_f32_tail.hip.inc).
   size_t ntail = 0, nmain = 0;
   const bool tail_ragged = kind == GemmKind::MfmaF16Edge && K <= (size_t(1) << 21) && N <= (size_t(1) << 22) && N % 8 == 0;
-  if ((kind == GemmKind::MfmaF16 || kind == GemmKind::MfmaF32 || tail_ragged) && !bt && !t128 && !split && batch == 1 &&
+  // full f16 tiles whose offsets inside a tile fit 32 bits: the operands go from memory straight into the LDS
+  // (kernels/gemm_f16_dma.hip.inc; B as it lies or transposed, single products and batches, whole and half tiles)
+  const bool dma_ok = kind == GemmKind::MfmaF16 && !t128 && !split && st_.fusion == FusionMode::Tree && st_.gemm_dma &&
+                      K <= (size_t(1) << 21) && N <= (size_t(1) << 22);
+  if ((kind == GemmKind::MfmaF16 || kind == GemmKind::MfmaF32 || tail_ragged) && (!bt || dma_ok) && !t128 && !split && batch == 1 &&
       st_.fusion == FusionMode::Tree && st_.gemm_tail) {
     nmain = tiles / cus * cus;
     ntail = tiles - nmain;
@@ -489,6 +496,8 @@ TensorData Resolver::run_matmul(const NodeP& n) {
                       (K == 64 || K == 128) && tiles * batch >= 4 * cus && cus % 8 == 0 && tiles * batch <= 0xffffffffull;
   // one column of 128-wide tiles over a long K, B small enough to stay in L2: the workgroups share no rows of A and
   // start their walk over K at different tiles (kernels/gemm_f16_t128.hip.inc, WKF_ROTK)
+  const bool dma = dma_ok && !shortk;
+  if (dma && !tail) nmain = tiles;
   const bool rotk = t128 && !split && N <= 128 && K >= 512 && K * N * dtype_size(a.dtype) <= (size_t(1) << 20);
   TensorData out = split ? alloc(slices_shape(slices), DType::F32, false) : alloc(out_shape, a.dtype, false);
   std::string sig = t128 ? std::string("gemm|gfx950|f16|mfma32x32x16|128x128x64|w2x2|edge") : gemm_signature(kind, a.dtype);
@@ -502,8 +511,10 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (bt) sig += "|bt";
   if (rotk) sig += "|rotk";
   if (shortk) sig += K == 64 ? "|whole K in LDS|nt1" : "|whole K in LDS|nt2";
-  if (tail) sig += "|last round in half tiles";  // (a ragged shape keeps "|edge" in front of it)
+  if (tail && !dma) sig += "|last round in half tiles";  // (a ragged shape keeps "|edge" in front of it)
+  if (dma) sig += "|direct to LDS";  // one binary for whole tiles and for a last round in half tiles
   wkf_kernel* k = kernel(sig, [&] {
+    if (dma) return std::string(bt ? "#define WKF_BT 1\n" : "") + kGemmF16Dma;
     if (tail && kind == GemmKind::MfmaF32) return std::string(kGemmF32Tail);
     if (tail) return std::string(tail_ragged ? "#define WKF_EDGEBUF 1\n" : "") + kGemmF16Tail;
     std::string src = bt ? "#define WKF_BT 1\n" : "";
@@ -525,7 +536,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (shortk) args.kchunk = uint32_t(batch);  // the kernel walks the tiles of every matrix itself
   std::vector<unsigned char> bytes(sizeof(args));
   memcpy(bytes.data(), &args, sizeof(args));
-  if (tail) {
+  if (tail || dma) {
     const uint32_t extra[2] = {uint32_t(nmain), uint32_t(ntail)};
     const size_t at = bytes.size();
     bytes.resize(at + sizeof(extra));
@@ -542,7 +553,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     if (r.grid[1] > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many rows for the generic kernel");
   } else {
     if (tiles > 0x7fffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
-    r.grid[0] = uint32_t(shortk ? cus : tail ? nmain + 2 * ntail : tiles);
+    r.grid[0] = uint32_t(shortk ? cus : (tail || dma) ? nmain + 2 * ntail : tiles);
     r.grid[1] = uint32_t(slices);
   }
   r.grid[2] = uint32_t(shortk ? 1 : batch);
@@ -552,6 +563,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (bt) d << " B^T";
   if (rotk) d << " K start rotated";
   if (shortk) d << ", whole K in LDS, one workgroup per compute unit walks the tiles";
+  if (dma) d << ", operands loaded straight into the LDS";
   if (split) d << " slices=" << slices;
   if (tail) d << ", last round: " << ntail << " tiles as " << 2 * ntail << " halves of 128 rows";
   if (batch > 1) d << " batch=" << batch;

@@ -118,6 +118,7 @@ Settings settings_for(wkf_device* dev) {
     if (const char* u = getenv("WKF_GEMM_SHORTK")) st.gemm_shortk = atoi(u) != 0;
     if (const char* u = getenv("WKF_MAP_TILE_VEC")) st.map_tile_vec = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_TAIL")) st.gemm_tail = atoi(u) != 0;
+    if (const char* u = getenv("WKF_GEMM_DMA")) st.gemm_dma = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_SPLIT")) st.row_split = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_TEAM")) st.row_team = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_STREAM_MIN_ROWS")) st.row_stream_min_rows = size_t(std::max(1ll, atoll(u)));
