@@ -88,6 +88,14 @@ int wkf_device_set_exact_math(wkf_device* dev, int exact);
 int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls);
 int wkf_device_row_team_fallbacks(wkf_device* dev, uint64_t* out);
 
+/* Maps over f16 as table lookups (no reference counterpart).  An element-wise kernel whose only operand is ONE dense
+ * f16 tensor and whose result is f16 computes a function of 16 bits.  When the fused chain is costly enough to
+ * make the kernel compute-bound (a transcendental function whose value feeds further arithmetic, say) and the
+ * tensor has at least `min_elements` elements (default 2^24; 0 = never), the 65536 values are computed once by
+ * the ordinary kernel over every bit pattern (kept per device, program and constants, the 32 most recent) and the
+ * data is streamed through a lookup in the LDS: the same bits as the ordinary kernel, at memory speed. */
+int wkf_device_set_map_table(wkf_device* dev, uint64_t min_elements);
+
 /* Per-kernel GPU timestamps (PerformanceQueries, src/query.rs:50-126: the reference
  * attaches one to every kernel).  On by default; a caller that only wants results can
  * switch the hipEvent pair per launch off. */

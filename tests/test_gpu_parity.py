@@ -1045,3 +1045,112 @@ def test_config5_gemm_full_size(gpu, name, m, n, k, dtype, tol):
     gemm_check(got, a, b, tol)
     if name == "f16-llama-mlp":  # 344 tiles on 256 compute units
         assert "last round: 88 tiles as 176 halves" in prod.kernels()[0].detail, prod.kernels()[0].detail
+
+
+# ---- maps over f16 as table lookups ------------------------------------------------------------------------------------
+
+def test_a_costly_map_over_one_f16_tensor_runs_as_a_table_lookup(gpu):
+    # An element-wise kernel over ONE dense f16 tensor with an f16 result is a function of 16 bits.  From a size on (the
+    # device setting; lowered here) a costly chain is computed once for all 65536 bit patterns by the ordinary kernel
+    # and the data goes through a lookup in the LDS.  The input holds every bit pattern (NaNs, infinities, denormals,
+    # both zeros) and a ragged tail; the result must be the ordinary kernel's, bit for bit, and the oracle's.
+    n = 3 * 65536 + 5
+    bits = np.concatenate([np.arange(65536, dtype=np.uint16), np.random.default_rng(3).integers(0, 65536, n - 65536).astype(np.uint16)])
+    x = bits.view(np.float16)
+    api = HipAPI(gpu)
+
+    def chains(t):
+        return [((t * 2.0) + 1.0).sin().exp(), t.silu(), (t.tanh() * 0.5 + 0.5).sqrt(), (t * t + 1.0).log().cos() / 3.0]
+
+    if gpu.is_planner:  # compile every kernel of this test, with and without tables, then skip
+        for least in (1 << 17, 0):
+            gpu.set_map_table(least)
+            try:
+                tx = api.tensor(x)
+                for p in chains(tx) + [((tx * 3.0) + 1.0).sin().exp(), ((tx.narrow(0, 8, 2 * 65536) * 2.0) + 1.0).sin().exp(),
+                                       ((tx.narrow(0, 3, 2 * 65536) * 2.0) + 1.0).sin().exp(), tx * 2.0 + 1.0, tx.sin().exp() + api.tensor(x)]:
+                    p.materialize()
+            finally:
+                gpu.set_map_table(1 << 24)
+        hip_values(api.tensor(x) * 2.0)
+    gpu.set_map_table(1 << 17)
+    try:
+        tx = api.tensor(x)
+        progs = chains(tx)
+        looked_up = [hip_values(p) for p in progs]
+        for p in progs:
+            details = [k.detail for k in p.kernels()]
+            assert "table lookup" in details[-1], details
+        # a second tensor, other constants: its own table; the same program again: the cached one (one launch)
+        again = ((tx * 2.0) + 1.0).sin().exp()
+        assert np.array_equal(hip_values(again).view(np.uint16), looked_up[0].view(np.uint16))
+        assert len(again.kernels()) == 1 and "table lookup" in again.kernels()[0].detail
+        other = ((tx * 3.0) + 1.0).sin().exp()
+        got_other = hip_values(other)
+        assert len(other.kernels()) == 2
+        # views: a dense slice that starts 16-byte aligned qualifies, a strided one and one off the grid do not
+        part = api.tensor(x).narrow(0, 8, 2 * 65536)
+        assert "table lookup" in [k.detail for k in ((part * 2.0) + 1.0).sin().exp().materialize().kernels()][-1]
+        off = api.tensor(x).narrow(0, 3, 2 * 65536)
+        assert "table lookup" not in [k.detail for k in ((off * 2.0) + 1.0).sin().exp().materialize().kernels()][-1]
+        assert np.array_equal(hip_values(((part * 2.0) + 1.0).sin().exp()).view(np.uint16), looked_up[0][8:8 + 2 * 65536].view(np.uint16))
+        # a cheap chain and a chain with two tensors stay ordinary kernels
+        assert "table lookup" not in (tx * 2.0 + 1.0).materialize().kernels()[0].detail
+        assert "table lookup" not in (tx.sin().exp() + api.tensor(x)).materialize().kernels()[0].detail
+    finally:
+        gpu.set_map_table(1 << 24)
+    gpu.set_map_table(0)
+    try:
+        plain = [hip_values(p) for p in chains(api.tensor(x))]
+        plain_other = hip_values(((api.tensor(x) * 3.0) + 1.0).sin().exp())
+    finally:
+        gpu.set_map_table(1 << 24)
+    for a, b in zip(looked_up, plain):
+        assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+    assert np.array_equal(got_other.view(np.uint16), plain_other.view(np.uint16))
+    with np.errstate(all="ignore"):
+        o = OTensor(x)
+        want = ((o * 2.0) + 1.0).sin().exp().to_numpy()
+    finite = np.isfinite(want)
+    assert np.array_equal(np.isnan(looked_up[0]), np.isnan(want))
+    assert np.array_equal(looked_up[0][finite].view(np.uint16), want[finite].view(np.uint16))
+
+
+def test_a_table_lookup_in_place_and_on_a_permuted_tensor(gpu):
+    # the operand may be overwritten (an intermediate nobody else holds: a product here), and input and output may share
+    # any permutation of dimensions as long as both are dense in it (the transposed product, updated in place)
+    a = data((512, 64), -1, 1, np.float16, 77)
+    b = data((64, 520), -1, 1, np.float16, 78)
+    api = HipAPI(gpu)
+
+    def run():
+        ta, tb = api.tensor(a), api.tensor(b)
+        straight = (ta.mat_mul(tb) * 2.0 + 1.0).sin().exp()
+        turned = (ta.mat_mul(tb).transpose(0, 1) * 2.0 + 1.0).sin().exp()
+        vals = hip_values_many([straight, turned])
+        return vals, [k.detail for k in straight.kernels()], [k.detail for k in turned.kernels()]
+
+    if gpu.is_planner:
+        gpu.set_map_table(0)
+        try:
+            ta, tb = api.tensor(a), api.tensor(b)
+            (ta.mat_mul(tb) * 2.0 + 1.0).sin().exp().materialize()
+            (ta.mat_mul(tb).transpose(0, 1) * 2.0 + 1.0).sin().exp().materialize()
+        finally:
+            gpu.set_map_table(1 << 24)
+    gpu.set_map_table(1 << 17)
+    try:
+        got, d0, d1 = run()
+    finally:
+        gpu.set_map_table(1 << 24)
+    assert "table lookup" in d0[-1] and "in_place" in d0[-1], d0
+    assert "table lookup" in d1[-1] and "in_place" in d1[-1], d1
+    gpu.set_map_table(0)
+    try:
+        want, e0, _ = run()
+    finally:
+        gpu.set_map_table(1 << 24)
+    assert "table lookup" not in e0[-1]
+    assert got[1].shape == (520, 512)
+    for g, w in zip(got, want):
+        assert np.array_equal(g.view(np.uint16), w.view(np.uint16))

@@ -621,6 +621,65 @@ std::string map_source(const MapSpec& s) {
   return o.str();
 }
 
+std::string map_table_signature() { return "maptable|gfx950|f16|b1024|u1"; }
+
+std::string map_table_source() {
+  std::ostringstream o;
+  o << kPrelude;
+  // One 16-byte vector per lane and round: 16 KiB in flight per compute unit is what a grid that stays on the chip
+  // streams fastest with (a plain copy of this shape: 42.8 us for 2 x 128 MiB with one vector, 46.7 with four)
+  o << R"WKF(
+typedef unsigned short u16;
+typedef u32 wkf_u4 __attribute__((ext_vector_type(4)));
+struct Args { const u16* in; u16* out; const u16* table; u32 nvec; u32 ntail; };
+extern "C" __global__ void __launch_bounds__(1024) WKF_ENTRY(const Args a) {
+  __shared__ __attribute__((aligned(16))) u16 lut[65536];
+  const u32 t = threadIdx.x;
+  const wkf_u4* const in = (const wkf_u4*)a.in;
+  wkf_u4* const out = (wkf_u4*)a.out;
+  const u32 step = gridDim.x * 1024u;
+  u32 w = blockIdx.x * 1024u + t;
+  // the first vector of the data is asked for before the table, so that it travels while the table is copied
+  wkf_u4 v = w < a.nvec ? __builtin_nontemporal_load(in + w) : (wkf_u4)(0u);
+#pragma unroll
+  for (int i = 0; i < 8; i++) ((wkf_u4*)lut)[t + i * 1024u] = ((const wkf_u4*)a.table)[t + i * 1024u];
+  __syncthreads();
+  if (blockIdx.x == 0 && t < a.ntail) a.out[size_t(a.nvec) * 8u + t] = lut[a.in[size_t(a.nvec) * 8u + t]];
+  while (w < a.nvec) {
+    wkf_u4 r;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+      const u32 d = v[e];
+      r[e] = u32(lut[d & 0xffffu]) | (u32(lut[d >> 16]) << 16);
+    }
+    const u32 w_now = w;
+    w += step;
+    // the next round's load goes out before this round's store
+    v = w < a.nvec ? __builtin_nontemporal_load(in + w) : (wkf_u4)(0u);
+    __builtin_nontemporal_store(r, out + w_now);
+  }
+}
+)WKF";
+  return o.str();
+}
+
+int program_cost(const Program& p) {
+  int cost = 0;
+  for (size_t i = 0; i < p.ins.size(); i++) {
+    const Op op = p.ins[i].op;
+    const bool interior = int(i) != p.result;
+    switch (op) {
+      case Op::Load: break;
+      case Op::DivC: case Op::RDivC: case Op::Div: cost += 3; break;
+      case Op::Sqrt: cost += 2; break;
+      case Op::Pow: cost += 10; break;
+      case Op::Sqr: case Op::Abs: case Op::Neg: cost += 1; break;
+      default: cost += is_unary_op(op) ? (interior ? 10 : 3) : 1; break;
+    }
+  }
+  return cost;
+}
+
 std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a) {
   const size_t N = s.in.size() + 1 + s.more_out.size();
   const size_t R = size_t(s.rank);

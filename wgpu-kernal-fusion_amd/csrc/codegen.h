@@ -64,6 +64,17 @@ constexpr int kMapTile = 64;
 
 std::string map_signature(const MapSpec& s);
 std::string map_source(const MapSpec& s);
+// out[i] = table[in[i]] over dense f16 data: any map whose only operand is one f16 tensor, with an f16 result, is a
+// function of 16 bits.  The table (65536 f16 values, 128 KiB, built once per program and constants by the map kernel
+// itself run over every bit pattern) is copied into the LDS of one 1024-lane workgroup per compute unit, which then
+// streams the data with 16-byte loads and stores and eight LDS reads per vector.  One binary serves every program.
+// Arguments: {const void* in; void* out; const void* table; u32 nvec (16-byte vectors); u32 ntail (elements after them)}.
+constexpr int kMapTableBlock = 1024;
+std::string map_table_signature();
+std::string map_table_source();
+// what a program costs per element in units of a plain arithmetic op (an estimate: a transcendental function whose value
+// feeds further arithmetic takes a correctly rounded core, about ten; the last one before the store about three)
+int program_cost(const Program& p);
 // Size in bytes of the argument block and the packer that fills it.
 struct MapArgs {
   std::vector<void*> ptrs;               // inputs..., out, further outputs...

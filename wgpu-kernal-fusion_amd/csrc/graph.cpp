@@ -4,6 +4,7 @@
 #include <functional>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <mutex>
 #include <set>
 #include <unordered_map>
@@ -295,6 +296,120 @@ uint64_t team_fallbacks(wkf_device* dev) {
   std::lock_guard<std::mutex> lock(g_team_mu);
   auto it = g_team.find(dev);
   return it == g_team.end() ? 0 : it->second.fallbacks;
+}
+
+namespace {
+// Lookup tables of map programs over f16 (try_map_table): per device the 65536 bit patterns as an input tensor and
+// the most recently used tables, keyed by program, math policy and constants.
+struct MapTables {
+  BufRef patterns;
+  std::vector<std::pair<std::string, BufRef>> tables;  // most recently used last
+};
+constexpr size_t kMaxMapTables = 32;  // 128 KiB each
+std::mutex g_tables_mu;
+std::unordered_map<wkf_device*, MapTables> g_tables;
+void tables_forget(wkf_device* dev) {
+  MapTables t;
+  {
+    std::lock_guard<std::mutex> lock(g_tables_mu);
+    auto it = g_tables.find(dev);
+    if (it == g_tables.end()) return;
+    t = std::move(it->second);
+    g_tables.erase(it);
+  }
+}  // the buffers are released here, outside the lock
+}  // namespace
+
+bool Resolver::try_map_table(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place) {
+  const size_t numel = out.layout.numel();
+  if (st_.fusion != FusionMode::Tree || st_.map_table_min == 0 || numel < std::max<size_t>(st_.map_table_min, 1u << 17) || noalloc_) return false;
+  if (in.size() != 1 || in[0].dtype != DType::F16 || out.dtype != DType::F16 || prog.result_dtype() != DType::F16) return false;
+  // both dense in the same order (any permutation of dimensions, as long as input and output share it), 16-byte aligned
+  if (in[0].layout.strides != out.layout.strides || in[0].layout.offset % 8 || out.layout.offset % 8) return false;
+  {
+    std::vector<std::pair<size_t, size_t>> dims_by_stride;
+    for (size_t d = 0; d < out.layout.shape.size(); d++)
+      if (out.layout.shape[d] != 1) dims_by_stride.push_back({out.layout.strides[d], out.layout.shape[d]});
+    std::sort(dims_by_stride.begin(), dims_by_stride.end());
+    size_t expect = 1;
+    for (const auto& ds : dims_by_stride) {
+      if (ds.first != expect) return false;
+      expect *= ds.second;
+    }
+  }
+  if (numel / 8 > 0xffffffffull || program_cost(prog) < 12 || wkf_device_closing_(dev_)) return false;
+  if ((in[0].layout.offset + numel) * 2 > wkf_buffer_size(in[0].buffer.get()) + 3 || (out.layout.offset + numel) * 2 > wkf_buffer_size(out.buffer.get()) + 3)
+    invalid("map kernel: a layout reaches past the end of its buffer");
+
+  const MathPolicy policy = st_.exact_math ? MathPolicy::Exact : st_.math_f32 ? MathPolicy::Folded : MathPolicy::Stored;
+  std::string key = prog.signature() + "|m" + std::to_string(int(policy)) + "|";
+  for (float c : prog.consts) {
+    char buf[16];
+    snprintf(buf, sizeof buf, "%08x,", __builtin_bit_cast(unsigned, c));
+    key += buf;
+  }
+  static const bool hooked = (wkf_add_destroy_hook_(&tables_forget), true);
+  (void)hooked;
+  BufRef patterns, table;
+  {
+    std::lock_guard<std::mutex> lock(g_tables_mu);
+    MapTables& mt = g_tables[dev_];
+    patterns = mt.patterns;
+    for (size_t i = 0; i < mt.tables.size(); i++)
+      if (mt.tables[i].first == key) {
+        table = mt.tables[i].second;
+        std::rotate(mt.tables.begin() + long(i), mt.tables.begin() + long(i) + 1, mt.tables.end());
+        break;
+      }
+  }
+  if (!table) {
+    if (!patterns) {
+      wkf_buffer* b = nullptr;
+      check(wkf_buffer_alloc(dev_, 65536 * 2, 0, &b));
+      patterns = BufRef(b);
+      std::vector<uint16_t> all(65536);
+      for (size_t i = 0; i < all.size(); i++) all[i] = uint16_t(i);
+      check(wkf_buffer_upload(b, 0, all.data(), all.size() * 2));
+    }
+    TensorData tin;
+    tin.device = dev_;
+    tin.buffer = patterns;
+    tin.layout = Layout::contiguous({65536});
+    tin.dtype = DType::F16;
+    TensorData tout = alloc({65536}, DType::F16, false);
+    launch_map(prog, {tin}, tout, false);  // the ordinary kernel (65536 elements are below any threshold), same policy
+    table = tout.buffer;
+    std::lock_guard<std::mutex> lock(g_tables_mu);
+    MapTables& mt = g_tables[dev_];
+    if (!mt.patterns) mt.patterns = patterns;
+    if (mt.tables.size() >= kMaxMapTables) mt.tables.erase(mt.tables.begin());
+    mt.tables.push_back({key, table});
+  }
+
+  const std::string sig = map_table_signature();
+  wkf_kernel* k = kernel(sig, [&] { return map_table_source(); });
+  struct {
+    const void* in;
+    void* out;
+    const void* table;
+    uint32_t nvec, ntail;
+  } args = {static_cast<const char*>(element_ptr(in[0])) + in[0].layout.offset * 2, static_cast<char*>(element_ptr(out)) + out.layout.offset * 2,
+            wkf_buffer_ptr(table.get()), uint32_t(numel / 8), uint32_t(numel % 8)};
+  std::vector<unsigned char> bytes(sizeof(args));
+  memcpy(bytes.data(), &args, sizeof(args));
+  wkf_props props;
+  check(wkf_device_props(dev_, &props));
+  LaunchRecord r;
+  r.kind = "map";
+  r.signature = sig;
+  r.in_place = in_place;
+  r.grid[0] = to_u32(std::min<size_t>(size_t(std::max(1, props.compute_units)), (numel / 8 + kMapTableBlock - 1) / kMapTableBlock), "grid");
+  r.block[0] = kMapTableBlock;
+  std::ostringstream d;
+  d << "shape=[" << numel << "] table lookup: 65536 values of " << prog.signature() << (in_place ? " in_place" : "");
+  r.detail = d.str();
+  record(std::move(r), k, bytes);
+  return true;
 }
 
 TensorData Resolver::alloc(const std::vector<size_t>& shape, DType dt, bool zero, bool result) {
@@ -1034,6 +1149,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
       invalid("operand shapes differ: " + dims(td.layout.shape) + " vs " + dims(shape));  // src/pair_wise.rs:92
   size_t numel = out.layout.numel();
   if (numel == 0) return;
+  if (more_out.empty() && try_map_table(prog, in, out, in_place)) return;
 
   // The order in which a map visits its elements is free: walk the dimensions in the order of the
   // OUTPUT's strides (largest first), so that a transposed output written in place is still one
@@ -1092,7 +1208,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   spec.rank = int(R);
   spec.vec = vec;
   spec.prog = prog;
-  spec.math = st_.exact_math ? MathPolicy::Exact : MathPolicy::Stored;
+  spec.math = st_.exact_math ? MathPolicy::Exact : st_.math_f32 ? MathPolicy::Folded : MathPolicy::Stored;
   // Inputs that run along another dimension than the output (a transposed operand): tiled kernel.
   spec.more_prog = more_prog;
   if (vec == 1 && R >= 2 && numel >= (size_t(1) << 16) && sp.strides[N - 1][R - 1] == 1 && sp.shape[R - 1] >= 16 &&

@@ -33,9 +33,11 @@ struct Settings {
   bool timing = true;             // record a hipEvent pair around every launch
   int map_unroll = 4;             // work items per thread in large map kernels (WKF_MAP_UNROLL overrides: 1, 2, 4, 8)
   bool exact_math = false;        // every transcendental through an f64 core (MathPolicy::Exact)
+  bool math_f32 = false;          // measurement only (WKF_MATH_F32=1): map kernels take the f32 library for every transcendental, outside the 2-ulp bound of fused chains; shows what the f64 cores cost
   size_t nontemporal_bytes = size_t(32) << 20;  // map kernels moving at least this much use streaming loads/stores
   int reduce_threads = 0;         // lanes per row in row reduces; 0 = chosen from the shape (WKF_REDUCE_THREADS overrides)
   int row_threads = 0;            // lanes per row in row kernels; 0 = chosen from the shape (WKF_ROW_THREADS overrides)
+  size_t map_table_min = size_t(1) << 24;  // fewest elements for which a costly map over ONE dense f16 tensor (f16 result) runs as a table lookup; 0 = never (WKF_MAP_TABLE_MIN)
   bool map_tile_vec = true;       // transposing map kernels move four elements per access where the layouts allow it (WKF_MAP_TILE_VEC=0: one)
   bool gemm_shortk = true;        // many full f16 tiles over K = 64 or 128: one workgroup per compute unit walks them (WKF_GEMM_SHORTK=0 turns it off)
   bool gemm_t128 = true;          // 128 x 128 tiles for f16 products that do not fill the chip with 256 x 256 ones (WKF_GEMM_T128=0 turns it off)
@@ -150,6 +152,11 @@ class Resolver {
   // `more_prog[j]` (over the same operands) is stored to `more_out[j]` by the same kernel.
   void launch_map(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place,
                   const std::vector<Program>& more_prog = {}, const std::vector<TensorData>& more_out = {});
+  // A map over one dense f16 tensor with an f16 result is a function of 16 bits: from map_table_min elements on, and
+  // when the program costs enough to make the kernel compute-bound, its 65536 values are computed once (by the ordinary
+  // kernel, over every bit pattern; kept per device, program and constants) and the data is streamed through a
+  // lookup in the LDS.  Bit-identical to the ordinary kernel by construction.  False: not applicable, nothing launched.
+  bool try_map_table(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
   void launch_map_tiled(MapSpec& spec, const Space& sp, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
   // `result`: the buffer receives the value of a reduce node (allocation-free mode: the caller's output tensor)
   TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero, bool result = false);

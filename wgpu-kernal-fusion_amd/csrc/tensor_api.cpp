@@ -119,6 +119,8 @@ Settings settings_for(wkf_device* dev) {
     if (const char* u = getenv("WKF_MAP_TILE_VEC")) st.map_tile_vec = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_TAIL")) st.gemm_tail = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_DMA")) st.gemm_dma = atoi(u) != 0;
+    if (const char* u = getenv("WKF_MATH_F32")) st.math_f32 = atoi(u) != 0;
+    if (const char* u = getenv("WKF_MAP_TABLE_MIN")) st.map_table_min = size_t(std::max(0ll, atoll(u)));
     if (const char* u = getenv("WKF_ROW_SPLIT")) st.row_split = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_TEAM")) st.row_team = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_STREAM_MIN_ROWS")) st.row_stream_min_rows = size_t(std::max(1ll, atoll(u)));
@@ -471,6 +473,15 @@ int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls) 
     g_settings[dev].row_team = enabled != 0;
     g_settings[dev].row_team_spin = (spin_polls & 0x7fffffffu) == 0 ? Settings().row_team_spin : (spin_polls & 0x7fffffffu);
     g_settings[dev].row_team_test_mute = (spin_polls >> 31) != 0;
+  });
+}
+
+int wkf_device_set_map_table(wkf_device* dev, uint64_t min_elements) {
+  return guarded([&] {
+    need(dev, "wkf_device_set_map_table");
+    settings_for(dev);
+    std::lock_guard<std::mutex> lock(g_settings_mu);
+    g_settings[dev].map_table_min = size_t(min_elements);
   });
 }
 
