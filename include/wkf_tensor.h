@@ -88,6 +88,13 @@ int wkf_device_set_exact_math(wkf_device* dev, int exact);
 int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls);
 int wkf_device_row_team_fallbacks(wkf_device* dev, uint64_t* out);
 
+/* Where a composite of the reference differs IN VALUE from what it means, this library computes what it means; with
+ * `enabled` != 0 tensors built afterwards on this device follow the reference's text instead.  One case today:
+ * layer_norm (src/composite/rms_norm.rs:13-14) broadcasts its weight with Tensor::broadcast, which puts the new
+ * dimension where the shapes first differ (src/map_layout.rs:69-77); for a square input (rows == hidden) that is
+ * position 1, so the weight is indexed by ROW.  Off by default (RMSNorm as meant: the weight along the last dimension). */
+int wkf_device_set_reference_compat(wkf_device* dev, int enabled);
+
 /* Maps over f16 as table lookups (no reference counterpart).  An element-wise kernel whose only operand is ONE dense
  * f16 tensor and whose result is f16 computes a function of 16 bits.  When the fused chain is costly enough to
  * make the kernel compute-bound (a transcendental function whose value feeds further arithmetic, say) and the

@@ -1154,3 +1154,34 @@ def test_a_table_lookup_in_place_and_on_a_permuted_tensor(gpu):
     assert got[1].shape == (520, 512)
     for g, w in zip(got, want):
         assert np.array_equal(g.view(np.uint16), w.view(np.uint16))
+
+
+# ---- the reference's text where it differs in value from what it means ---------------------------------------------------
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+def test_layer_norm_as_the_reference_text_reads_on_square_inputs(gpu, dtype):
+    # src/composite/rms_norm.rs:13-14 broadcasts the weight with Tensor::broadcast (src/map_layout.rs:69-77): on a
+    # square input the weight is indexed by row.  Off by default (RMSNorm as meant); with the device's
+    # reference-compat flag the library follows the text, in both fusion modes, and non-square inputs do not change.
+    sq = data((96, 96), -2, 2, dtype, 31)
+    rect = data((64, 96), -2, 2, dtype, 32)
+    w = data((96,), 0.5, 1.5, dtype, 33)
+    api = HipAPI(gpu)
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == np.float32 else dict(rtol=2e-3, atol=1e-3)
+    meant = hip_values(api.tensor(sq).layer_norm(api.tensor(w), 1e-5))
+    assert np.allclose(meant, OTensor(sq).layer_norm(OTensor(w), 1e-5).to_numpy(), **tol)
+    want_sq = OTensor(sq).layer_norm_as_written(OTensor(w), 1e-5).to_numpy()
+    want_rect = OTensor(rect).layer_norm(OTensor(w), 1e-5).to_numpy()
+    assert not np.allclose(want_sq, meant, **tol)  # the two readings differ on this input
+    gpu.set_reference_compat(True)
+    try:
+        for mode in (1, 0):
+            gpu.set_fusion(mode)
+            got_sq, got_rect = hip_values_many([api.tensor(sq).layer_norm(api.tensor(w), 1e-5), api.tensor(rect).layer_norm(api.tensor(w), 1e-5)])
+            assert np.allclose(got_sq, want_sq, **tol), mode
+            assert np.allclose(got_rect, want_rect, **tol), mode
+    finally:
+        gpu.set_fusion(1)
+        gpu.set_reference_compat(False)
+    again = hip_values(api.tensor(sq).layer_norm(api.tensor(w), 1e-5))
+    assert np.array_equal(again, meant)

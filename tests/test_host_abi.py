@@ -619,6 +619,29 @@ def test_reduce_into_plans_without_allocating_and_refuses_the_rest(wkf):
     dev.close()
 
 
+def test_reference_compat_changes_only_the_square_layer_norm(wkf):
+    # the flag is per device and acts when the tensor is built: for a square input the weight's broadcast lands on
+    # dimension 1, as the reference's text reads, so along a row the weight is ONE value (axis stride 0 in the row
+    # kernel's signature) instead of a row of values (axis stride 1); a non-square input plans the same kernel either way
+    dev = wkf.Device.planner()
+    T = wkf.Tensor
+    w = T.new(dev, np.ones((8,), dtype=np.float32))
+    sq, rect = T.new(dev, np.ones((8, 8), dtype=np.float32)), T.new(dev, np.ones((4, 8), dtype=np.float32))
+
+    def plan(x):
+        t = x.layer_norm(w, 1e-5).materialize()
+        return [k.signature for k in t.kernels()]
+
+    meant, rect_meant = plan(sq), plan(rect)
+    dev.set_reference_compat(True)
+    written, rect_written = plan(sq), plan(rect)
+    dev.set_reference_compat(False)
+    assert len(meant) == len(written) == 1
+    assert "|in:f32a1,f32a1,|" in meant[0] and "|in:f32a1,f32a0,|" in written[0]
+    assert rect_written == rect_meant and plan(sq) == meant
+    dev.close()
+
+
 def test_a_timer_outlives_its_device_handle(wkf):
     # A timer keeps its device alive like a buffer does (its events go back to that device's pool): destroying the
     # device first and the timer afterwards must find the device still there, and the device goes with the timer.

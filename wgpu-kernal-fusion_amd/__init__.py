@@ -40,7 +40,7 @@ EXPORTS = [
     "wkf_buffer_download", "wkf_buffer_copy", "wkf_module_get", "wkf_module_find", "wkf_module_stats", "wkf_device_alloc_stats", "wkf_launch",
     "wkf_timer_create", "wkf_timer_destroy", "wkf_timer_begin", "wkf_timer_end", "wkf_timer_elapsed_ns",
     "wkf_last_error",
-    "wkf_device_set_fusion", "wkf_device_get_fusion", "wkf_device_set_exact_math", "wkf_device_set_row_teams", "wkf_device_row_team_fallbacks", "wkf_device_set_map_table", "wkf_device_set_timing", "wkf_tensor_new", "wkf_tensor_clone", "wkf_tensor_free",
+    "wkf_device_set_fusion", "wkf_device_get_fusion", "wkf_device_set_exact_math", "wkf_device_set_row_teams", "wkf_device_row_team_fallbacks", "wkf_device_set_map_table", "wkf_device_set_reference_compat", "wkf_device_set_timing", "wkf_tensor_new", "wkf_tensor_clone", "wkf_tensor_free",
     "wkf_tensor_rank", "wkf_tensor_shape", "wkf_tensor_dtype", "wkf_tensor_scalar_op", "wkf_tensor_unary_op",
     "wkf_tensor_cast", "wkf_tensor_binary_op", "wkf_tensor_reduce", "wkf_tensor_reduce_into", "wkf_tensor_mat_mul", "wkf_tensor_slice",
     "wkf_tensor_transpose", "wkf_tensor_broadcast", "wkf_tensor_narrow", "wkf_tensor_resize",
@@ -152,6 +152,7 @@ def load():
     lib.wkf_device_set_row_teams.argtypes = [c_void_p, c_int, ctypes.c_uint32]
     lib.wkf_device_row_team_fallbacks.argtypes = [c_void_p, POINTER(c_uint64)]
     lib.wkf_device_set_map_table.argtypes = [c_void_p, c_uint64]
+    lib.wkf_device_set_reference_compat.argtypes = [c_void_p, c_int]
     lib.wkf_module_stats.argtypes = [c_void_p, POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]
     lib.wkf_device_alloc_stats.argtypes = [c_void_p, POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64), POINTER(c_uint64)]
     lib.wkf_buffer_alloc.argtypes = [c_void_p, c_size_t, c_int, POINTER(c_void_p)]
@@ -287,6 +288,11 @@ class Device:
         """Rows held in the registers of several workgroups that wait for each other (one launch, one read); see
         wkf_device_set_row_teams.  spin_polls = 0 keeps the default bound of the wait."""
         _check(self._lib.wkf_device_set_row_teams(self._h, 1 if enabled else 0, int(spin_polls)))
+
+    def set_reference_compat(self, enabled):
+        """Composites follow the reference's text where it differs in value from what it means (layer_norm on square
+        inputs: the weight indexed by row); see wkf_device_set_reference_compat."""
+        _check(self._lib.wkf_device_set_reference_compat(self._h, 1 if enabled else 0))
 
     def set_map_table(self, min_elements):
         """Fewest elements for which a costly map over one dense f16 tensor runs as a table lookup (0: never); see

@@ -367,7 +367,7 @@ NodeP n_silu(const NodeP& x) {
 }
 
 // `layer_norm` = RMSNorm computed in f32, src/composite/rms_norm.rs:8-15.
-NodeP n_layer_norm(const NodeP& x, const NodeP& weight, float eps) {
+NodeP n_layer_norm(const NodeP& x, const NodeP& weight, float eps, bool as_written) {
   if (x->shape.size() != 2 || weight->shape.size() != 1) invalid("layer_norm: expects a rank-2 tensor and a rank-1 weight");
   if (weight->shape[0] != x->shape[1]) invalid("layer_norm: the weight length must equal the last dimension");
   if (weight->dtype != x->dtype) invalid("layer_norm: dtype mismatch");
@@ -378,6 +378,12 @@ NodeP n_layer_norm(const NodeP& x, const NodeP& weight, float eps) {
   // The reference spells these two broadcasts with Tensor::broadcast, which picks
   // the wrong dimension for the weight when rows == hidden (src/map_layout.rs:69-75);
   // the dimensions are named here.
+  // the dimensions are named here.  `as_written` (wkf_device_set_reference_compat) takes Tensor::broadcast for
+  // both, as the reference's text does: on a square input the weight is then indexed by row.
+  if (as_written) {
+    NodeP x_normed = n_pair_wise(f32_self, n_broadcast(rms, x->shape), Op::Div);
+    return n_pair_wise(n_cast(x_normed, x->dtype), n_broadcast(weight, x->shape), Op::Mul);
+  }
   NodeP x_normed = n_pair_wise(f32_self, n_broadcast_at(rms, 1, hidden), Op::Div);
   return n_pair_wise(n_cast(x_normed, x->dtype), n_broadcast_at(weight, 0, x->shape[0]), Op::Mul);
 }
@@ -473,6 +479,15 @@ int wkf_device_set_row_teams(wkf_device* dev, int enabled, uint32_t spin_polls) 
     g_settings[dev].row_team = enabled != 0;
     g_settings[dev].row_team_spin = (spin_polls & 0x7fffffffu) == 0 ? Settings().row_team_spin : (spin_polls & 0x7fffffffu);
     g_settings[dev].row_team_test_mute = (spin_polls >> 31) != 0;
+  });
+}
+
+int wkf_device_set_reference_compat(wkf_device* dev, int enabled) {
+  return guarded([&] {
+    need(dev, "wkf_device_set_reference_compat");
+    settings_for(dev);
+    std::lock_guard<std::mutex> lock(g_settings_mu);
+    g_settings[dev].reference_compat = enabled != 0;
   });
 }
 
@@ -730,7 +745,7 @@ int wkf_tensor_layer_norm(const wkf_tensor* t, const wkf_tensor* weight, float e
     need(t, "wkf_tensor_layer_norm");
     need(weight, "wkf_tensor_layer_norm");
     need(out, "wkf_tensor_layer_norm");
-    *out = wrap(t->dev, n_layer_norm(t->node, weight->node, eps));
+    *out = wrap(t->dev, n_layer_norm(t->node, weight->node, eps, settings_for(t->dev).reference_compat));
   });
 }
 
