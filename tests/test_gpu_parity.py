@@ -9,6 +9,8 @@ Tolerances (stated where they are used):
   reductions (sum, product) and what is built on them              1e-5 relative
   max / min                                                        bit-exact
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -952,6 +954,49 @@ def test_a_few_rows_against_a_very_wide_weight_keep_their_slice_of_a_small(gpu):
     first = t.kernels()[0]
     assert "|skinny_bt|valu|m16|c1024" in first.signature and "slices=2" in first.detail, (first.signature, first.detail)
     gemm_check(got, a, np.ascontiguousarray(w.T), 1e-3)
+
+
+FLEX_CONFIGS = ["2,3,4,1", "2,3,4,3", "2,3,3,2", "2,2,2,1", "2,2,2,4", "1,3,4,1", "1,3,4,2", "1,4,4,1", "1,2,5,2", "1,2,5,4", "2,4,3,1", "2,4,2,2"]
+
+
+@pytest.mark.parametrize("config", FLEX_CONFIGS)
+def test_every_tile_of_the_flexible_f16_kernel(wkf, config, monkeypatch):
+    # The f16 kernel that loads its operands straight into the LDS takes tiles of 64 NI x 64 NJ, a ring of LDS stages and K
+    # slices chosen per shape.  Here every configuration the planner may choose (and two more) is forced on a device of its
+    # own (the override is read when a device is created): ragged M and N, a single K step, fewer steps than stages, B
+    # as it lies and transposed, and a batch; all against the f64 product.
+    monkeypatch.setenv("WKF_GEMM_FLEX", config)
+    planner_run = os.environ.get("WKF_TEST_PLAN_ONLY") == "1"
+    dev = wkf.Device.planner() if planner_run else wkf.Device.new(0)
+    try:
+        slices = int(config.split(",")[3])
+        rng = np.random.default_rng(sum(int(v) * 7 ** i for i, v in enumerate(config.split(","))))
+        cases = [(300, 1000, 512, False, ()), (77, 200, 64, False, ()), (512, 776, 1024, True, ()), (129, 136, 128, False, ()),
+                 (64, 192, 2048, True, ()), (200, 264, 256, False, (3,))]
+        for m, n, k, bt, lead in cases:
+            a = rng.standard_normal(lead + (m, k)).astype(np.float16)
+            b = rng.standard_normal(lead + ((n, k) if bt else (k, n))).astype(np.float16)
+            ta, tb = wkf.Tensor.new(dev, a), wkf.Tensor.new(dev, b)
+            r = len(lead) + 2
+            t = ta.mat_mul(tb.transpose(r - 2, r - 1) if bt else tb)
+            if planner_run:
+                t.materialize()
+                continue
+            got = t.to_numpy()
+            first = t.kernels()[0]
+            assert "operands loaded straight into the LDS" in first.detail and f"{64 * int(config[0])}x{64 * int(config[2])} tiles" in first.detail, first.detail
+            if slices > 1 and not lead and k // slices >= 64:
+                assert "slices=" in first.detail and len(t.kernels()) == 2
+            bm = np.swapaxes(b, -1, -2) if bt else b
+            if lead:
+                for z in range(lead[0]):
+                    gemm_check(got[z], a[z], np.ascontiguousarray(bm[z]), 1e-2)
+            else:
+                gemm_check(got, a, np.ascontiguousarray(bm), 1e-2)
+    finally:
+        dev.close()
+    if planner_run:
+        pytest.skip("plan-only device: kernels compiled, nothing computed")
 
 
 # (batch dimensions, m, n, k, B given as a transposed view): attention-like products, ragged ones, tiny ones

@@ -456,7 +456,7 @@ def test_f16_column_max_with_a_post_op_compiles(wkf, planner):
 def test_mat_mul_kernel_choice(wkf, planner):
     def detail(m, n, k, dtype):
         t = _x(wkf, planner, (m, k), dtype).mat_mul(_x(wkf, planner, (k, n), dtype, seed=1))
-        assert _kinds(t) == ["gemm"]
+        assert _kinds(t) in (["gemm"], ["gemm", "red_col"])  # (K in slices: the f32 partial sums are folded by a second launch)
         return t.kernels()[0].detail
 
     # full f16 tiles: the operands go from memory straight into the LDS (whole tiles and a last round in half tiles)
@@ -470,7 +470,11 @@ def test_mat_mul_kernel_choice(wkf, planner):
     assert detail(300, 260, 68, np.float32).endswith("mfma 256x256 tiles edge")
     assert detail(4096, 4352, 64, np.float32).endswith("mfma 256x256 tiles, last round: 16 tiles as 32 halves of 128 rows")
     # f16 products whose large tiles would fill at most half of the chip take 128 x 128 tiles, two workgroups per compute unit
-    assert detail(512, 256, 128, np.float16).endswith("mfma 128x128 tiles")
+    # (K a multiple of 64: a tile of 64 NI x 64 NJ chosen by a cost model, operands loaded straight into the LDS; else 128 x 128)
+    assert detail(512, 256, 128, np.float16).endswith("mfma 64x192 tiles, operands loaded straight into the LDS, 4 stages")
+    assert detail(512, 11008, 4096, np.float16).endswith("mfma 128x192 tiles, operands loaded straight into the LDS, 4 stages")
+    assert detail(128, 4096, 4096, np.float16).endswith("mfma 64x128 tiles, operands loaded straight into the LDS, 5 stages slices=4")
+    assert detail(512, 264, 136, np.float16).endswith("mfma 128x128 tiles")
     assert detail(300, 264, 72, np.float16).endswith("mfma 128x128 tiles")
     assert detail(1024, 11008, 512, np.float16).endswith("mfma 256x256 tiles, operands loaded straight into the LDS")
     # unaligned rows or tiny problems: the generic kernel
@@ -492,7 +496,7 @@ def test_mat_mul_kernel_choice(wkf, planner):
     # x * W^T for a dense W [N, K] needs no copy: the MFMA kernels read W as it lies ...
     w = _x(wkf, planner, (512, 256), np.float16, seed=2)
     t = _x(wkf, planner, (256, 256), np.float16).mat_mul(w.transpose(0, 1))
-    assert _kinds(t) == ["gemm"] and t.kernels()[0].detail.endswith("B^T") and "|bt" in t.kernels()[0].signature
+    assert _kinds(t) == ["gemm"] and "tiles B^T" in t.kernels()[0].detail and "|bt" in t.kernels()[0].signature
     big_w = _x(wkf, planner, (4096, 256), np.float16, seed=2)
     t = _x(wkf, planner, (4096, 256), np.float16).mat_mul(big_w.transpose(0, 1))
     assert _kinds(t) == ["gemm"] and "B^T" in t.kernels()[0].detail and t.kernels()[0].signature.endswith("|bt|direct to LDS")
@@ -525,7 +529,7 @@ def test_batched_mat_mul_is_one_launch(wkf, planner):
     k = _x(wkf, planner, (8, 512, 128), np.float16, seed=1)
     scores = q.mat_mul(k.transpose(1, 2))                      # q k^T per head: k is read as it lies
     assert scores.shape() == (8, 512, 512) and _kinds(scores) == ["gemm"]
-    assert scores.kernels()[0].detail.endswith("B^T batch=8") and "|bt" in scores.kernels()[0].signature
+    assert "tiles B^T" in scores.kernels()[0].detail and scores.kernels()[0].detail.endswith("batch=8") and "|bt" in scores.kernels()[0].signature
     v = _x(wkf, planner, (8, 512, 128), np.float16, seed=2)
     out = scores.softmax_last_dim().mat_mul(v)
     assert out.shape() == (8, 512, 128) and _kinds(out) == ["gemm", "row", "gemm"]
@@ -547,12 +551,12 @@ def test_batched_mat_mul_is_one_launch(wkf, planner):
     # (128 columns: a narrow B, whose rows the lanes of a block share among themselves)
     assert "skinny narrow slices" in o1.kernels()[-2].detail and o1.kernels()[-2].detail.endswith("batch=8")
     assert o1.kernels()[-2].signature.endswith("|skinny|m1|v8|narrow16")
-    # the same binaries as a single product: no new module for the batch
+    # the same kernel source as a single product (the tile may differ: it is chosen for the number of workgroups)
     before = planner.module_stats()
     _x(wkf, planner, (3, 256, 64), np.float16).mat_mul(_x(wkf, planner, (3, 64, 256), np.float16, seed=1)).materialize()
     _x(wkf, planner, (256, 64), np.float16).mat_mul(_x(wkf, planner, (64, 256), np.float16, seed=1)).materialize()
     after = planner.module_stats()
-    assert (after["compiled"] + after["disk_hits"]) - (before["compiled"] + before["disk_hits"]) <= 1
+    assert (after["compiled"] + after["disk_hits"]) - (before["compiled"] + before["disk_hits"]) <= 2
     for bad_a, bad_b in (((2, 4, 8), (3, 8, 4)), ((2, 4, 8), (8, 4)), ((2, 4, 8), (2, 7, 4)), ((8,), (8,))):
         with pytest.raises(wkf.WkfError) as e:
             _x(wkf, planner, bad_a, np.float32).mat_mul(_x(wkf, planner, bad_b, np.float32, seed=1))
@@ -724,6 +728,12 @@ def test_gemm_kernels_use_no_scratch_memory(tmp_path):
         "    mm(4000, 4001, 136, dt, True)      # rows of C off the 16-byte grid: the ragged kernel that addresses with pointers\n"
         "    mm(3, 5, 7, dt)                    # the generic kernel\n"
         "    mm(64, 64, 32, dt, lead=(3,))\n"
+        "import os\n"
+        "for cfg in ('2,3,4,1', '2,3,4,3', '2,3,3,2', '2,2,2,1', '2,2,2,4', '1,3,4,1', '1,3,4,2', '1,4,4,1', '1,2,5,2', '1,2,5,4'):\n"
+        "    os.environ['WKF_GEMM_FLEX'] = cfg     # every tile of the flexible f16 kernel, forced on a device of its own\n"
+        "    dev = w.Device.planner()\n"
+        "    mm(300, 1000, 2048, np.float16); mm(300, 1000, 2048, np.float16, True)\n"
+        "del os.environ['WKF_GEMM_FLEX']\n"
     )
     env = dict(os.environ, WKF_CACHE_DIR=str(tmp_path))
     subprocess.run([sys.executable, "-c", script], check=True, env=env, timeout=900)
@@ -734,9 +744,10 @@ def test_gemm_kernels_use_no_scratch_memory(tmp_path):
                 continue
             checked += 1
             assert k[".private_segment_fixed_size"] == 0 and not k[".uses_dynamic_stack"], (k[".name"], k[".private_segment_fixed_size"])
-            assert k[".vgpr_spill_count"] == 0 and k[".sgpr_spill_count"] == 0, (k[".name"], k[".vgpr_spill_count"], k[".sgpr_spill_count"])
+            # (a scalar register parked in a lane of a vector register outside the loop costs nothing and touches no memory)
+            assert k[".vgpr_spill_count"] == 0 and k[".sgpr_spill_count"] <= 8, (k[".name"], k[".vgpr_spill_count"], k[".sgpr_spill_count"])
             assert k[".vgpr_count"] <= 512
-    assert checked >= 22, f"only {checked} GEMM kernels were compiled: the shapes above no longer reach the variants"
+    assert checked >= 40, f"only {checked} GEMM kernels were compiled: the shapes above no longer reach the variants"
 
 
 def test_team_row_kernels_fit_four_workgroups_per_compute_unit(tmp_path):

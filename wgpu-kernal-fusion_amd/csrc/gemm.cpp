@@ -41,6 +41,9 @@ const char* const kGemmF16T128 =
 const char* const kGemmF16Dma =
 #include "kernels/gemm_f16_dma.hip.inc"
     ;
+const char* const kGemmF16Flex =
+#include "kernels/gemm_f16_flex.hip.inc"
+    ;
 const char* const kGemmF16Tail =
 #include "kernels/gemm_f16_tail.hip.inc"
     ;
@@ -90,6 +93,48 @@ std::string gemm_source(GemmKind kind, DType dt) {
       return std::string("#define WKF_T ") + (dt == DType::F32 ? "float" : "_Float16") + "\n" + kGemmGeneric;
   }
   return "";
+}
+
+// Chooses the tile of the flexible f16 kernel for [M x K] x [K x N] on `cus` compute units: 32-row and 32-column blocks
+// per wave (the tile is 64 ni x 64 nj), LDS stages and K slices, by a cost model fitted to a sweep on MI355X
+// (21 shapes [64..1024] x {4096, 11008} x {4096, 11008}, 14 configurations; mean error 8 %).  A step of a lone
+// workgroup on a compute unit takes `step_us`; two workgroups that share a compute unit (128 x 128 tiles in two
+// stages) take 0.79 of running one after the other; every further round costs 7.5 us, the fold of K slices 8.5 us.
+struct FlexChoice { int ni, nj, ns; size_t slices; };
+static double flex_model_us(const FlexChoice& c, size_t M, size_t N, size_t K, size_t batch, size_t cus) {
+  static const double step_us[3][5] = {{0, 0, 0, 0, 0}, {0, 0, 0.281, 0.414, 0.566}, {0, 0, 0.427, 0.635, 0.737}};
+  const size_t tiles = ((M + 64 * c.ni - 1) / (64 * c.ni)) * ((N + 64 * c.nj - 1) / (64 * c.nj)) * batch;
+  size_t kc = ((K + c.slices - 1) / c.slices + 63) / 64 * 64;
+  const size_t S = (K + kc - 1) / kc, steps = kc / 64;
+  const size_t per_cu = 160 / (size_t(c.ns) * 8 * (c.ni + c.nj)) >= 2 ? 2 : 1;
+  const size_t load = (tiles * S + cus - 1) / cus;  // workgroups per compute unit
+  const double s = step_us[c.ni][c.nj] * (c.ns == 2 ? 1.6 : 1.0);
+  double t = 3.4;
+  if (per_cu == 1) t += double(load) * steps * s + double(load - 1) * 7.5;
+  else {
+    const size_t rounds = (load + 1) / 2;
+    t += double(load / 2) * steps * s * 2 * 0.79 + double(load % 2) * steps * s + double(rounds - 1) * 7.5;
+  }
+  if (S > 1) t += 8.5;
+  return t;
+}
+static void pick_flex(size_t M, size_t N, size_t K, size_t batch, size_t cus, int* ni, int* nj, int* ns, size_t* slices) {
+  static const FlexChoice candidates[] = {{2, 3, 4, 1}, {2, 3, 4, 3}, {2, 3, 3, 2}, {2, 2, 2, 1}, {2, 2, 2, 2}, {2, 2, 2, 4}, {1, 3, 4, 1}, {1, 3, 4, 2},
+                                          {1, 3, 4, 4}, {1, 4, 4, 1}, {1, 2, 5, 2}, {1, 2, 5, 4}};
+  *ni = 0;
+  double best = 1e30;
+  for (const FlexChoice& c : candidates) {
+    if (batch > 1 && c.slices > 1) continue;
+    if (c.slices > 1 && (K / c.slices < 512 || c.slices * M * N * 4 > (M * K + K * N) * 2)) continue;  // partial sums stay below the operands' bytes
+    const double t = flex_model_us(c, M, N, K, batch, cus);
+    if (t < best) {
+      best = t;
+      *ni = c.ni;
+      *nj = c.nj;
+      *ns = c.ns;
+      *slices = c.slices;
+    }
+  }
 }
 
 TensorData Resolver::run_matmul(const NodeP& n) {
@@ -456,6 +501,73 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // (its loads take 32-bit byte offsets into a matrix: each operand matrix stays under 2 GiB)
   const bool t128 = mfma && a.dtype == DType::F16 && st_.fusion == FusionMode::Tree && st_.gemm_t128 &&
                     ((tiles256 * batch * 2 <= cus && !long_k_in_slices) || pad128 * 20 <= pad256 * 11) && M * K < (size_t(1) << 30) && K * N < (size_t(1) << 30);
+  // Tiles of 64 NI x 64 NJ with the operands loaded straight into the LDS (kernels/gemm_f16_flex.hip.inc), for products
+  // that the 256 x 256 tile would spread badly over the chip.  WKF_GEMM_FLEX="ni,nj,stages,slices" forces a shape.
+  // (rows of C 16-byte aligned, N % 8 == 0: the kernel stores whole 16-byte vectors)
+  if (mfma && a.dtype == DType::F16 && st_.fusion == FusionMode::Tree && K % 64 == 0 && N % 8 == 0 && M * K < (size_t(1) << 30) &&
+      K * N < (size_t(1) << 30)) {
+    int ni = 0, nj = 0, ns = 0;
+    size_t S = 1;
+    bool forced = false;
+    if (const char* f = getenv("WKF_GEMM_FLEX")) {
+      unsigned long long sl = 1;
+      forced = sscanf(f, "%d,%d,%d,%llu", &ni, &nj, &ns, &sl) == 4 && ni >= 1 && ni <= 2 && nj >= 2 && nj <= 4 && ns >= 2 &&
+               size_t(ns) * 8 * (ni + nj) <= 160 && sl >= 1;
+      S = size_t(sl);
+      if (!forced) ni = 0;
+    }
+    // where the 128 x 128 tile would be taken (a few hundred rows against a wide weight, small batches), except one
+    // column of tiles over a long K against a small B, which keeps that kernel's rotated walk over K
+    const bool one_column = N <= 128 && K >= 512 && K * N * dtype_size(a.dtype) <= (size_t(1) << 20);
+    if (!forced && st_.gemm_flex && t128 && !one_column) {
+      S = 1;
+      pick_flex(M, N, K, batch, cus, &ni, &nj, &ns, &S);
+    }
+    if (ni > 0 && batch > 1) S = 1;
+    size_t kc = 0;
+    if (ni > 0 && S > 1) {
+      kc = ((K + S - 1) / S + 63) / 64 * 64;
+      S = (K + kc - 1) / kc;
+    }
+    if (ni > 0) {
+      const bool sp = S > 1;
+      const size_t bm = 64 * size_t(ni), bn = 64 * size_t(nj);
+      const size_t ftiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn);
+      if (ftiles > 0x7fffffffull || S > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
+      TensorData fout = sp ? alloc(slices_shape(S), DType::F32, false) : alloc(out_shape, a.dtype, false);
+      std::string fsig = "gemm|gfx950|f16|mfma32x32x16|" + std::to_string(bm) + "x" + std::to_string(bn) + "x64|w2x2|direct to LDS|stages" + std::to_string(ns);
+      if (sp) fsig += "|splitk";
+      if (bt) fsig += "|bt";
+      wkf_kernel* fk = kernel(fsig, [&] {
+        return "#define WKF_NI " + std::to_string(ni) + "\n#define WKF_NJ " + std::to_string(nj) + "\n#define WKF_NS " + std::to_string(ns) + "\n" +
+               (sp ? "#define WKF_SPLITK 1\n" : "") + (bt ? "#define WKF_BT 1\n" : "") + kGemmF16Flex;
+      });
+      struct {
+        const void* a;
+        const void* b;
+        void* c;
+        uint32_t m, n, k, kchunk;
+      } fargs = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(fout.buffer.get()),
+                 uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(kc)};
+      std::vector<unsigned char> fbytes(sizeof(fargs));
+      memcpy(fbytes.data(), &fargs, sizeof(fargs));
+      LaunchRecord r;
+      r.kind = "gemm";
+      r.signature = fsig;
+      r.block[0] = 256;
+      r.grid[0] = uint32_t(ftiles);
+      r.grid[1] = uint32_t(S);
+      r.grid[2] = uint32_t(batch);
+      std::ostringstream d;
+      d << "m=" << M << " n=" << N << " k=" << K << " mfma " << bm << "x" << bn << " tiles" << (bt ? " B^T" : "") << ", operands loaded straight into the LDS, "
+        << ns << " stages";
+      if (sp) d << " slices=" << S;
+      if (batch > 1) d << " batch=" << batch;
+      r.detail = d.str();
+      record(std::move(r), fk, fbytes);
+      return sp ? fold_slices(fout) : fout;
+    }
+  }
   const size_t tile = t128 ? 128 : 256;
   const size_t tiles = ((M + tile - 1) / tile) * ((N + tile - 1) / tile);
   const size_t slots = t128 ? 2 * cus : cus;  // workgroups the chip holds at once

@@ -43,6 +43,7 @@ struct Settings {
   bool gemm_shortk = true;        // many full f16 tiles over K = 64 or 128: one workgroup per compute unit walks them (WKF_GEMM_SHORTK=0 turns it off)
   bool gemm_t128 = true;          // 128 x 128 tiles for f16 products that do not fill the chip with 256 x 256 ones (WKF_GEMM_T128=0 turns it off)
   bool gemm_dma = true;           // full f16 256 x 256 tiles load their operands from memory straight into the LDS (WKF_GEMM_DMA=0: through registers)
+  bool gemm_flex = true;          // f16 products that the 256 x 256 tile spreads badly over the chip take tiles of 64 NI x 64 NJ chosen per shape (WKF_GEMM_FLEX=0 turns it off; "ni,nj,stages,slices" forces one)
   bool gemm_tail = true;          // a partly filled last round of f16 tiles runs as half tiles (WKF_GEMM_TAIL=0 turns it off)
   int skinny_tr_rows = 0;         // fewest rows of A for the MFMA decode kernel on row-major B; 0 = chosen (WKF_SKINNY_TR_ROWS overrides)
   int skinny_blocks = 0;          // workgroups the decode-sized mat_mul kernels aim for; 0 = chosen (WKF_SKINNY_BLOCKS overrides)
