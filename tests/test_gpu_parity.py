@@ -1116,7 +1116,7 @@ def test_a_costly_map_over_one_f16_tensor_runs_as_a_table_lookup(gpu):
                                        ((tx.narrow(0, 3, 2 * 65536) * 2.0) + 1.0).sin().exp(), tx * 2.0 + 1.0, tx.sin().exp() + api.tensor(x)]:
                     p.materialize()
             finally:
-                gpu.set_map_table(1 << 24)
+                gpu.set_map_table(1 << 25)
         hip_values(api.tensor(x) * 2.0)
     gpu.set_map_table(1 << 17)
     try:
@@ -1143,13 +1143,13 @@ def test_a_costly_map_over_one_f16_tensor_runs_as_a_table_lookup(gpu):
         assert "table lookup" not in (tx * 2.0 + 1.0).materialize().kernels()[0].detail
         assert "table lookup" not in (tx.sin().exp() + api.tensor(x)).materialize().kernels()[0].detail
     finally:
-        gpu.set_map_table(1 << 24)
+        gpu.set_map_table(1 << 25)
     gpu.set_map_table(0)
     try:
         plain = [hip_values(p) for p in chains(api.tensor(x))]
         plain_other = hip_values(((api.tensor(x) * 3.0) + 1.0).sin().exp())
     finally:
-        gpu.set_map_table(1 << 24)
+        gpu.set_map_table(1 << 25)
     for a, b in zip(looked_up, plain):
         assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
     assert np.array_equal(got_other.view(np.uint16), plain_other.view(np.uint16))
@@ -1182,19 +1182,19 @@ def test_a_table_lookup_in_place_and_on_a_permuted_tensor(gpu):
             (ta.mat_mul(tb) * 2.0 + 1.0).sin().exp().materialize()
             (ta.mat_mul(tb).transpose(0, 1) * 2.0 + 1.0).sin().exp().materialize()
         finally:
-            gpu.set_map_table(1 << 24)
+            gpu.set_map_table(1 << 25)
     gpu.set_map_table(1 << 17)
     try:
         got, d0, d1 = run()
     finally:
-        gpu.set_map_table(1 << 24)
+        gpu.set_map_table(1 << 25)
     assert "table lookup" in d0[-1] and "in_place" in d0[-1], d0
     assert "table lookup" in d1[-1] and "in_place" in d1[-1], d1
     gpu.set_map_table(0)
     try:
         want, e0, _ = run()
     finally:
-        gpu.set_map_table(1 << 24)
+        gpu.set_map_table(1 << 25)
     assert "table lookup" not in e0[-1]
     assert got[1].shape == (520, 512)
     for g, w in zip(got, want):

@@ -925,6 +925,7 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
     streamed = true;
     ragged = false;
     NV = std::max<size_t>(1, std::min<size_t>(4, 8 / std::max<size_t>(1, K)));  // vectors in flight per lane and operand
+    if (st_.row_stream_vectors > 0) NV = size_t(st_.row_stream_vectors);
     if (nrows >= st_.row_stream_min_rows) {
       T = 1024;
     } else {

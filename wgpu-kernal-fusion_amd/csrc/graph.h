@@ -38,7 +38,7 @@ struct Settings {
   size_t nontemporal_bytes = size_t(32) << 20;  // map kernels moving at least this much use streaming loads/stores
   int reduce_threads = 0;         // lanes per row in row reduces; 0 = chosen from the shape (WKF_REDUCE_THREADS overrides)
   int row_threads = 0;            // lanes per row in row kernels; 0 = chosen from the shape (WKF_ROW_THREADS overrides)
-  size_t map_table_min = size_t(1) << 24;  // fewest elements for which a costly map over ONE dense f16 tensor (f16 result) runs as a table lookup; 0 = never (WKF_MAP_TABLE_MIN)
+  size_t map_table_min = size_t(1) << 25;  // fewest elements for which a costly map over ONE dense f16 tensor (f16 result) runs as a table lookup; 0 = never (WKF_MAP_TABLE_MIN)
   bool map_tile_vec = true;       // transposing map kernels move four elements per access where the layouts allow it (WKF_MAP_TILE_VEC=0: one)
   bool gemm_shortk = true;        // many full f16 tiles over K = 64 or 128: one workgroup per compute unit walks them (WKF_GEMM_SHORTK=0 turns it off)
   bool gemm_t128 = true;          // 128 x 128 tiles for f16 products that do not fill the chip with 256 x 256 ones (WKF_GEMM_T128=0 turns it off)
@@ -52,6 +52,7 @@ struct Settings {
   bool row_team = true;              // rows too long for a block's registers that fit those of up to 256 blocks: one launch, the row read once, the blocks of a row exchange their folds and wait for each other (WKF_ROW_TEAM=0 turns it off)
   uint32_t row_team_spin = 1u << 20; // polls a lane of such a kernel may spend waiting before it gives up (the read-back then computes the tensor again without teams)
   bool row_team_test_mute = false;   // tests of that path: a kernel variant in which part 0 of every row stays silent
+  int row_stream_vectors = 0;        // vectors per lane and operand in flight in the kernels that stream rows longer than a block's registers; 0 = chosen (WKF_ROW_STREAM_VECTORS)
   size_t row_stream_min_rows = 256;  // fewest rows for the one-launch kernel that streams rows longer than a block's registers (WKF_ROW_STREAM_MIN_ROWS)
 };
 

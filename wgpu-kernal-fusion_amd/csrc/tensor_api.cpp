@@ -124,6 +124,10 @@ Settings settings_for(wkf_device* dev) {
     if (const char* u = getenv("WKF_MAP_TABLE_MIN")) st.map_table_min = size_t(std::max(0ll, atoll(u)));
     if (const char* u = getenv("WKF_ROW_SPLIT")) st.row_split = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_TEAM")) st.row_team = atoi(u) != 0;
+    if (const char* u = getenv("WKF_ROW_STREAM_VECTORS")) {
+      int v = atoi(u);
+      if (v >= 1 && v <= 8) st.row_stream_vectors = v;
+    }
     if (const char* u = getenv("WKF_ROW_STREAM_MIN_ROWS")) st.row_stream_min_rows = size_t(std::max(1ll, atoll(u)));
     if (const char* u = getenv("WKF_SKINNY_TR_ROWS")) {
       int v = atoi(u);
