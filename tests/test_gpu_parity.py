@@ -1016,8 +1016,13 @@ BATCH_SHAPES = [((4,), 256, 256, 64, False), ((3,), 100, 72, 40, False), ((2, 3)
 # many full tiles over K = 64 or 128: one workgroup per compute unit walks the tiles of the whole batch
 BATCH_SHAPES += [((3,), 4, 72, 300, False), ((64,), 1, 64, 1024, False)]  # decode rows against a narrow B
 BATCH_SHAPES += [((5,), 2, 300, 264, True), ((40,), 1, 1000, 72, True), ((2, 3), 4, 260, 4096, True)]  # decode rows on the vector ALUs
-BATCH_SHAPES += [((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)]
-WHOLE_K = {((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False)}
+BATCH_SHAPES += [((16,), 2048, 2048, 128, True), ((4,), 4096, 4096, 64, False), ((2, 2), 4096, 4096, 128, False), ((13,), 2304, 2304, 64, True), ((1030,), 256, 256, 128, False),
+                 ((16,), 2048, 2048, 192, True), ((17,), 2048, 2048, 256, False), ((5,), 4096, 3840, 192, False)]
+WHOLE_K = {((4,), 4096, 4096, 64, False), ((13,), 2304, 2304, 64, True)}
+# many full tiles over K = 128 to 256: a tile's stores leave under the next tile's MFMAs (a tile count that is no multiple
+# of 8 or of the compute units, every K, B as it lies and transposed)
+STREAMED = {((16,), 2048, 2048, 128, True), ((2, 2), 4096, 4096, 128, False), ((1030,), 256, 256, 128, False), ((16,), 2048, 2048, 192, True),
+            ((17,), 2048, 2048, 256, False), ((5,), 4096, 3840, 192, False)}
 ROTATED = {((2,), 2048, 128, 2048, False), ((4,), 640, 100, 1096, False), ((3,), 384, 128, 2048, True), ((2, 2), 130, 72, 520, False),
            ((8,), 512, 128, 512, False)}
 
@@ -1048,6 +1053,8 @@ def test_batched_mat_mul(gpu, lead, m, n, k, bt, dtype, tol):
     gemm_of = lambda t: [kk for kk in t.kernels() if kk.kind == "gemm"][0].detail  # noqa: E731
     if (lead, m, n, k, bt) in WHOLE_K and dtype == np.float16:
         assert "whole K in LDS" in gemm_of(prod), gemm_of(prod)
+    if (lead, m, n, k, bt) in STREAMED and dtype == np.float16:
+        assert "stores under the next tile" in gemm_of(prod), gemm_of(prod)
     if (lead, m, n, k, bt) in ROTATED and dtype == np.float16:
         assert "K start rotated" in gemm_of(prod), gemm_of(prod)
     if not bt and "skinny" not in prod.kernels()[0].detail and "slices" not in gemm_of(one):

@@ -728,6 +728,8 @@ def test_gemm_kernels_use_no_scratch_memory(tmp_path):
         "    mm(4000, 4001, 136, dt, True)      # rows of C off the 16-byte grid: the ragged kernel that addresses with pointers\n"
         "    mm(3, 5, 7, dt)                    # the generic kernel\n"
         "    mm(64, 64, 32, dt, lead=(3,))\n"
+        "    for k in (128, 192, 256):          # many full tiles over a short K: a tile's stores under the next tile's MFMAs (f16)\n"
+        "        mm(2048, 2048, k, dt, True, lead=(16,)); mm(2048, 2048, k, dt, False, lead=(16,))\n"
         "import os\n"
         "for cfg in ('2,3,4,1', '2,3,4,3', '2,3,3,2', '2,2,2,1', '2,2,2,4', '1,3,4,1', '1,3,4,2', '1,4,4,1', '1,2,5,2', '1,2,5,4'):\n"
         "    os.environ['WKF_GEMM_FLEX'] = cfg     # every tile of the flexible f16 kernel, forced on a device of its own\n"

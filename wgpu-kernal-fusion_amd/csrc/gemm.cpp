@@ -44,6 +44,9 @@ const char* const kGemmF16Dma =
 const char* const kGemmF16Flex =
 #include "kernels/gemm_f16_flex.hip.inc"
     ;
+const char* const kGemmF16Stream =
+#include "kernels/gemm_f16_stream.hip.inc"
+    ;
 const char* const kGemmF16Tail =
 #include "kernels/gemm_f16_tail.hip.inc"
     ;
@@ -604,11 +607,16 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   // Many full tiles over K = 64 or 128 (attention scores, a low-rank update): what bounds them is the stores of C.  One
   // workgroup per compute unit walks the tiles of the whole batch with the next tile's operands in flight under the
   // current tile's MFMAs and stores (kernels/gemm_f16_shortk.hip.inc).
-  const bool shortk = kind == GemmKind::MfmaF16 && !t128 && !split && !tail && st_.fusion == FusionMode::Tree && st_.gemm_shortk &&
-                      (K == 64 || K == 128) && tiles * batch >= 4 * cus && cus % 8 == 0 && tiles * batch <= 0xffffffffull;
+  const bool many_tiles = kind == GemmKind::MfmaF16 && !t128 && !split && !tail && st_.fusion == FusionMode::Tree && tiles * batch >= 4 * cus &&
+                          cus % 8 == 0 && tiles * batch <= 0xffffffffull;
+  // ... and over K = 128 to 256 the stores of a tile are issued under the MFMAs of the next (kernels/gemm_f16_stream.hip.inc)
+  // (its buffer resources cover one whole tensor of the batch each: 32-bit byte offsets)
+  const bool stream = many_tiles && st_.gemm_stream && (K == 128 || K == 192 || K == 256) && batch * M * K < (size_t(1) << 30) &&
+                      batch * K * N < (size_t(1) << 30) && batch * M * N < (size_t(1) << 30);
+  const bool shortk = many_tiles && !stream && st_.gemm_shortk && (K == 64 || K == 128);
   // one column of 128-wide tiles over a long K, B small enough to stay in L2: the workgroups share no rows of A and
   // start their walk over K at different tiles (kernels/gemm_f16_t128.hip.inc, WKF_ROTK)
-  const bool dma = dma_ok && !shortk;
+  const bool dma = dma_ok && !shortk && !stream;
   if (dma && !tail) nmain = tiles;
   const bool rotk = t128 && !split && N <= 128 && K >= 512 && K * N * dtype_size(a.dtype) <= (size_t(1) << 20);
   TensorData out = split ? alloc(slices_shape(slices), DType::F32, false) : alloc(out_shape, a.dtype, false);
@@ -623,6 +631,11 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (bt) sig += "|bt";
   if (rotk) sig += "|rotk";
   if (shortk) sig += K == 64 ? "|whole K in LDS|nt1" : "|whole K in LDS|nt2";
+  if (stream) {
+    sig += "|stores under the next tile|nk" + std::to_string(K / 64);
+    if (const char* v = getenv("WKF_GEMM_STREAM_IMM")) sig += std::string("|imm") + v;
+    if (const char* v = getenv("WKF_GEMM_STREAM_EARLY")) sig += std::string("|early") + v;
+  }
   if (tail && !dma) sig += "|last round in half tiles";  // (a ragged shape keeps "|edge" in front of it)
   if (dma) sig += "|direct to LDS";  // one binary for whole tiles and for a last round in half tiles
   wkf_kernel* k = kernel(sig, [&] {
@@ -632,6 +645,12 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     std::string src = bt ? "#define WKF_BT 1\n" : "";
     if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (rotk ? "#define WKF_ROTK 1\n" : "") + kGemmF16T128;
     if (shortk) return src + (K == 64 ? "#define WKF_NT 1\n" : "#define WKF_NT 2\n") + kGemmF16ShortK;
+    if (stream) {
+      std::string defs = "#define WKF_NK " + std::to_string(K / 64) + "\n";
+      if (const char* v = getenv("WKF_GEMM_STREAM_IMM")) defs += "#define WKF_IMM " + std::to_string(std::max(1, std::min(3, atoi(v)))) + "\n";
+      if (const char* v = getenv("WKF_GEMM_STREAM_EARLY")) defs += "#define WKF_EARLY " + std::to_string(atoi(v) != 0 ? 1 : 0) + "\n";
+      return src + defs + kGemmF16Stream;
+    }
     if (ragged16) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (edge_ptr ? "#define WKF_EDGE 1\n" : "#define WKF_EDGEBUF 1\n") + kGemmF16;
     if (!split) return src + gemm_source(kind, a.dtype);
     const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;
@@ -645,7 +664,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     uint32_t m, n, k, kchunk;
   } args = {wkf_buffer_ptr(a.buffer.get()), wkf_buffer_ptr(b.buffer.get()), wkf_buffer_ptr(out.buffer.get()),
             uint32_t(M), uint32_t(N), uint32_t(K), uint32_t(kchunk)};
-  if (shortk) args.kchunk = uint32_t(batch);  // the kernel walks the tiles of every matrix itself
+  if (shortk || stream) args.kchunk = uint32_t(batch);  // the kernel walks the tiles of every matrix itself
   std::vector<unsigned char> bytes(sizeof(args));
   memcpy(bytes.data(), &args, sizeof(args));
   if (tail || dma) {
@@ -665,10 +684,10 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     if (r.grid[1] > 65535) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many rows for the generic kernel");
   } else {
     if (tiles > 0x7fffffffull) throw Error(WKF_ERR_UNSUPPORTED, "mat_mul: too many tiles");
-    r.grid[0] = uint32_t(shortk ? cus : (tail || dma) ? nmain + 2 * ntail : tiles);
+    r.grid[0] = uint32_t((shortk || stream) ? cus : (tail || dma) ? nmain + 2 * ntail : tiles);
     r.grid[1] = uint32_t(slices);
   }
-  r.grid[2] = uint32_t(shortk ? 1 : batch);
+  r.grid[2] = uint32_t((shortk || stream) ? 1 : batch);
   std::ostringstream d;
   d << "m=" << M << " n=" << N << " k=" << K << (kind == GemmKind::Generic ? " generic" : t128 ? " mfma 128x128 tiles" : " mfma 256x256 tiles");
   if (!t128 && (kind == GemmKind::MfmaF16Edge || kind == GemmKind::MfmaF32Edge)) d << " edge";
@@ -676,6 +695,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (rotk) d << " K start rotated";
   if (shortk) d << ", whole K in LDS, one workgroup per compute unit walks the tiles";
   if (dma) d << ", operands loaded straight into the LDS";
+  if (stream) d << ", one workgroup per compute unit walks the tiles, a tile's stores under the next tile's MFMAs";
   if (split) d << " slices=" << slices;
   if (tail) d << ", last round: " << ntail << " tiles as " << 2 * ntail << " halves of 128 rows";
   if (batch > 1) d << " batch=" << batch;

@@ -41,6 +41,7 @@ struct Settings {
   size_t map_table_min = size_t(1) << 25;  // fewest elements for which a costly map over ONE dense f16 tensor (f16 result) runs as a table lookup; 0 = never (WKF_MAP_TABLE_MIN)
   bool map_tile_vec = true;       // transposing map kernels move four elements per access where the layouts allow it (WKF_MAP_TILE_VEC=0: one)
   bool gemm_shortk = true;        // many full f16 tiles over K = 64 or 128: one workgroup per compute unit walks them (WKF_GEMM_SHORTK=0 turns it off)
+  bool gemm_stream = true;        // many full f16 tiles over K = 128 to 256: one workgroup per compute unit walks them and a tile's stores leave under the next tile's MFMAs (WKF_GEMM_STREAM=0 turns it off)
   bool gemm_t128 = true;          // 128 x 128 tiles for f16 products that do not fill the chip with 256 x 256 ones (WKF_GEMM_T128=0 turns it off)
   bool gemm_dma = true;           // full f16 256 x 256 tiles load their operands from memory straight into the LDS (WKF_GEMM_DMA=0: through registers)
   bool gemm_flex = true;          // f16 products that the 256 x 256 tile spreads badly over the chip take tiles of 64 NI x 64 NJ chosen per shape (WKF_GEMM_FLEX=0 turns it off; "ni,nj,stages,slices" forces one)

@@ -116,6 +116,7 @@ Settings settings_for(wkf_device* dev) {
     }
     if (const char* u = getenv("WKF_GEMM_T128")) st.gemm_t128 = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_SHORTK")) st.gemm_shortk = atoi(u) != 0;
+    if (const char* u = getenv("WKF_GEMM_STREAM")) st.gemm_stream = atoi(u) != 0;
     if (const char* u = getenv("WKF_MAP_TILE_VEC")) st.map_tile_vec = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_TAIL")) st.gemm_tail = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_DMA")) st.gemm_dma = atoi(u) != 0;
