@@ -787,6 +787,48 @@ def yardsticks(w, dev, seeded, which, launches):
                                          + (f"{nblk} persistent blocks" if persist else "one chunk per block"),
                                  "us": round(us, 1), "GB/s": round(moved / us * 1e-3)})
         out["streams_1GiB"] = rows
+        # The same plain kernels at the sizes of the small BASELINE configurations (a launch's ramp and tail weigh more the
+        # less it moves): 32 MiB -> 32 MiB (RMSNorm, RoPE), 64 MiB -> 64 MiB (config 1), 256 MiB read (config 2).  Each launch
+        # takes the next piece of the 1 GiB buffers, so nothing is served from a cache.  `kernel_us` is the median of the
+        # dispatches' own begin-to-end times (what a profiler's kernel trace shows), `batch_us` one event pair around 50
+        # launches back to back.
+        sized = []
+        for mode, name, piece in ((0, "copy", 32 << 20), (0, "copy", 64 << 20), (1, "read-only", 256 << 20)):
+            for wg, u in ((256, 4), (256, 8), (1024, 8)):
+                defs = f"#define MODE {mode}\n#define WG {wg}\n#define U {u}\n#define NTL 1\n#define NTS 1\n#define PERSIST 0\n"
+                k = kernel(f"yardstick|stream|{mode}|{wg}|{u}|1|1|0", defs + STREAM_SRC, "wkf_stream")
+                n4 = piece // 16
+                grid, block = (c_uint32 * 3)(n4 // (wg * u), 1, 1), (c_uint32 * 3)(wg, 1, 1)
+                pieces = n // piece
+                packed = [struct.pack("PPQP", lib.wkf_buffer_ptr(src_b) + i * piece, lib.wkf_buffer_ptr(dst_b) + i * piece, n4,
+                                      lib.wkf_buffer_ptr(src2_b)) for i in range(pieces)]
+                turn = [0]
+
+                def launch(timer=None):
+                    a = packed[turn[0] % pieces]
+                    turn[0] += 1
+                    return lib.wkf_launch(dev._h, k, grid, block, 0, a, len(a), timer)
+
+                batch = _raw_timed(lib, dev, launch, 50, 20)
+                timers = []
+                for _ in range(30):
+                    t = c_void_p()
+                    assert lib.wkf_timer_create(dev._h, byref(t)) == 0
+                    assert launch(t) == 0
+                    timers.append(t)
+                dev.sync()
+                each = []
+                for t in timers:
+                    ns = ctypes.c_uint64()
+                    assert lib.wkf_timer_elapsed_ns(t, byref(ns)) == 0
+                    each.append(ns.value / 1e3)
+                    lib.wkf_timer_destroy(t)
+                moved = piece * (2 if mode == 0 else 1)
+                med = float(np.median(each))
+                sized.append({"what": f"{name} kernel, {piece >> 20} MiB per stream, {wg} threads, {u} x 16 B per lane, non-temporal on",
+                              "moved_MiB": moved >> 20, "kernel_us": round(med, 2), "kernel_min_us": round(min(each), 2), "batch_us": round(batch, 2),
+                              "GB/s_kernel": round(moved / med * 1e-3), "GB/s_batch": round(moved / batch * 1e-3)})
+        out["streams_sized"] = sized
         for name in ("copy", "read-only", "write-only", "two reads + one write"):
             best = max((r for r in rows if r["what"].startswith(name)), key=lambda r: r["GB/s"])
             out["best_" + name.replace("-", "_").replace(" + ", "_").replace(" ", "_")] = best

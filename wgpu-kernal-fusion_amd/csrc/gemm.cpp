@@ -631,11 +631,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
   if (bt) sig += "|bt";
   if (rotk) sig += "|rotk";
   if (shortk) sig += K == 64 ? "|whole K in LDS|nt1" : "|whole K in LDS|nt2";
-  if (stream) {
-    sig += "|stores under the next tile|nk" + std::to_string(K / 64);
-    if (const char* v = getenv("WKF_GEMM_STREAM_IMM")) sig += std::string("|imm") + v;
-    if (const char* v = getenv("WKF_GEMM_STREAM_EARLY")) sig += std::string("|early") + v;
-  }
+  if (stream) sig += "|stores under the next tile|nk" + std::to_string(K / 64);
   if (tail && !dma) sig += "|last round in half tiles";  // (a ragged shape keeps "|edge" in front of it)
   if (dma) sig += "|direct to LDS";  // one binary for whole tiles and for a last round in half tiles
   wkf_kernel* k = kernel(sig, [&] {
@@ -645,12 +641,7 @@ TensorData Resolver::run_matmul(const NodeP& n) {
     std::string src = bt ? "#define WKF_BT 1\n" : "";
     if (t128) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (rotk ? "#define WKF_ROTK 1\n" : "") + kGemmF16T128;
     if (shortk) return src + (K == 64 ? "#define WKF_NT 1\n" : "#define WKF_NT 2\n") + kGemmF16ShortK;
-    if (stream) {
-      std::string defs = "#define WKF_NK " + std::to_string(K / 64) + "\n";
-      if (const char* v = getenv("WKF_GEMM_STREAM_IMM")) defs += "#define WKF_IMM " + std::to_string(std::max(1, std::min(3, atoi(v)))) + "\n";
-      if (const char* v = getenv("WKF_GEMM_STREAM_EARLY")) defs += "#define WKF_EARLY " + std::to_string(atoi(v) != 0 ? 1 : 0) + "\n";
-      return src + defs + kGemmF16Stream;
-    }
+    if (stream) return src + "#define WKF_NK " + std::to_string(K / 64) + "\n" + kGemmF16Stream;
     if (ragged16) return src + (split ? "#define WKF_SPLITK 1\n" : "") + (edge_ptr ? "#define WKF_EDGE 1\n" : "#define WKF_EDGEBUF 1\n") + kGemmF16;
     if (!split) return src + gemm_source(kind, a.dtype);
     const GemmKind base = a.dtype == DType::F16 ? GemmKind::MfmaF16Edge : GemmKind::MfmaF32Edge;

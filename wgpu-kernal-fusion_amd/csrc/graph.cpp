@@ -870,9 +870,12 @@ bool Resolver::launch_row(RowBuild& rb, const Program* final_in, std::vector<Ten
   const size_t max_nv = size_t(16 * (Vmax / V));
   // Lanes per row, measured on MI355X: two 16-byte vectors per lane up to 256 lanes (softmax over 2048
   // floats: 169 us with 256 lanes, 173 with 64; RMSNorm over 4096: 15.9 us with 256, 17.2 with 128), more
-  // lanes only when a lane would otherwise hold more than 16 vectors.
+  // lanes only when a lane would otherwise hold more than 16 vectors.  An f16 row of up to 256 vectors stays in ONE wave
+  // (four vectors per lane, no fold through the LDS and no barrier: f16 softmax over 2048: 87.1 us with 128 lanes, 83.8
+  // with 64; f32 rows of 1024 lose 2 % that way and keep 128 lanes).
   const int T_wide = [&] {
     int t = std::min(256, pow2_ceil((nvec + 1) / 2));
+    if (nvec <= 256 && Vmax == 8) t = std::min(t, 64);
     while (t < 1024 && nvec > size_t(t) * 16) t *= 2;
     return t;
   }();
