@@ -367,6 +367,12 @@ def build_workloads(w, dev, seeded, which, with_cpu=False):
                                   HBM_PEAK_GBS, "f16")
         out["f16_map"] = Workload("f16: exp(sin(x*2+1)), f16 [8192,8192]", [[((x * 2.0) + 1.0).sin().exp()] for x in xs],
                                   2 * 8192 * 8192 * 2, "GB/s", HBM_PEAK_GBS, "f16")
+        # config 3 on f16: silu(a) depends on one operand only and is looked up in a table inside the fused kernel
+        b16 = T.new(dev, seeded(3, 2, (4096,), "normal", dtype=F16, std=0.02)).broadcast([1024, 4096]).broadcast([32, 1024, 4096])
+        ab = [(T.new(dev, seeded(3, 4 * r, (32, 1024, 4096), "uniform", dtype=F16)), T.new(dev, seeded(3, 4 * r + 1, (32, 1024, 4096), "uniform", dtype=F16)))
+              for r in range(2)]
+        out["f16_c3"] = Workload("f16: silu(a)*(b+bias), f16 [32,1024,4096]", [[a_.silu() * (b_ + b16)] for a_, b_ in ab],
+                                 3 * 32 * 1024 * 4096 * 2 + 4096 * 2, "GB/s", HBM_PEAK_GBS, "f16")
         x32 = [T.new(dev, seeded(2, r, (8192, 8192), "normal")) for r in range(2)]
         out["f16_cast"] = Workload("cast f32 -> f16, [8192,8192]", [[x.cast(w.F16)] for x in x32], 8192 * 8192 * 6, "GB/s",
                                    HBM_PEAK_GBS, "f32->f16")

@@ -262,7 +262,7 @@ class Tensor {
   }
   template <int R2>
   Tensor<R2, D> broadcast(const std::array<size_t, size_t(R2)>& out_shape) const {
-    static_assert(R2 >= R, "broadcast cannot drop dimensions");
+    static_assert(R2 == R + 1, "broadcast adds one leading dimension (src/map_layout.rs:69-77)");
     wkf_tensor* o = nullptr;
     check(wkf_tensor_broadcast(h_, R2, out_shape.data(), &o));
     return Tensor<R2, D>::adopt(o);

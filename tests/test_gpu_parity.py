@@ -1143,12 +1143,14 @@ def test_a_costly_map_over_one_f16_tensor_runs_as_a_table_lookup(gpu):
         # views: a dense slice that starts 16-byte aligned qualifies, a strided one and one off the grid do not
         part = api.tensor(x).narrow(0, 8, 2 * 65536)
         assert "table lookup" in [k.detail for k in ((part * 2.0) + 1.0).sin().exp().materialize().kernels()][-1]
+        # (one off the 16-byte grid goes through the general map kernel, which then looks the whole chain up as well)
         off = api.tensor(x).narrow(0, 3, 2 * 65536)
-        assert "table lookup" not in [k.detail for k in ((off * 2.0) + 1.0).sin().exp().materialize().kernels()][-1]
+        off_chain = ((off * 2.0) + 1.0).sin().exp()
+        assert np.array_equal(hip_values(off_chain).view(np.uint16), looked_up[0][3:3 + 2 * 65536].view(np.uint16))
+        assert "vec=1" in off_chain.kernels()[-1].detail and "table lookup" in off_chain.kernels()[-1].detail
         assert np.array_equal(hip_values(((part * 2.0) + 1.0).sin().exp()).view(np.uint16), looked_up[0][8:8 + 2 * 65536].view(np.uint16))
-        # a cheap chain and a chain with two tensors stay ordinary kernels
+        # a cheap chain stays an ordinary kernel
         assert "table lookup" not in (tx * 2.0 + 1.0).materialize().kernels()[0].detail
-        assert "table lookup" not in (tx.sin().exp() + api.tensor(x)).materialize().kernels()[0].detail
     finally:
         gpu.set_map_table(1 << 25)
     gpu.set_map_table(0)
@@ -1166,6 +1168,69 @@ def test_a_costly_map_over_one_f16_tensor_runs_as_a_table_lookup(gpu):
     finite = np.isfinite(want)
     assert np.array_equal(np.isnan(looked_up[0]), np.isnan(want))
     assert np.array_equal(looked_up[0][finite].view(np.uint16), want[finite].view(np.uint16))
+
+
+def test_a_costly_value_of_one_f16_operand_inside_a_larger_map_is_looked_up(gpu):
+    # silu(a) inside silu(a) * (b + bias), tanh(a) inside a * tanh(a) + b: a value that depends on ONE f16 operand is a
+    # function of 16 bits whatever else the kernel does.  The planner cuts the costliest such value out of the fused
+    # program, fills a table with it (the cut program run over all 65536 bit patterns, its last op evaluated as the
+    # interior op it was) and the kernel, 1024 lanes per compute unit around the table in the LDS, looks it up.  Results
+    # must equal the ordinary kernel's bit for bit and the oracle's.
+    rows, cols = 260, 1032   # ragged: the last chunk of 1024 work items is partly filled
+    a = data((rows, cols), -6, 6, np.float16, 501)
+    a.reshape(-1)[:65536] = np.arange(65536, dtype=np.uint16).view(np.float16)   # every bit pattern, NaNs included
+    b = data((rows, cols), -2, 2, np.float16, 502)
+    bias = data((cols,), -1, 1, np.float16, 503)
+    c32 = data((rows, cols), -2, 2, np.float32, 504)
+    wide = data((rows, 2 * cols), -2, 2, np.float16, 505)
+    api = HipAPI(gpu)
+
+    def graphs(T, ta, tb, tbias, tc, twide):
+        strided = twide.slice([(0, rows), (8, 8 + cols)])
+        return {
+            "silu(a)*(b+bias)": ta.silu() * (tb + tbias.broadcast([rows, cols])),
+            "tanh(a)*b": ta.tanh() * tb,
+            "a*tanh(a)+b": ta * ta.tanh() + tb,
+            "sin(a)*b+cos(a)": ta.sin() * tb + ta.cos(),                      # two values of one operand: one is looked up
+            "exp(a/2)+strided": (ta / 2.0).exp() + strided,                   # a strided second operand
+            "tanh(a) as f32 * c": ta.tanh().cast(0) * tc,            # the value is f16, the kernel's result f32
+            "log(1+a*a)-b*3": ((ta * ta) + 1.0).log() - (tb * 3.0),           # a pair-wise op inside the value
+        }
+
+    def run(least):
+        gpu.set_map_table(least)
+        try:
+            g = graphs(api, api.tensor(a), api.tensor(b), api.tensor(bias), api.tensor(c32), api.tensor(wide))
+            vals = {k: hip_values(t) for k, t in g.items()}
+            return vals, {k: [kk.detail for kk in t.kernels()] for k, t in g.items()}
+        finally:
+            gpu.set_map_table(1 << 25)
+
+    if gpu.is_planner:  # compile every kernel of this test, with and without tables, then skip
+        for least in (1 << 17, 0):
+            gpu.set_map_table(least)
+            try:
+                for t in graphs(api, api.tensor(a), api.tensor(b), api.tensor(bias), api.tensor(c32), api.tensor(wide)).values():
+                    t.materialize()
+            finally:
+                gpu.set_map_table(1 << 25)
+    got, details = run(1 << 17)
+    for k, d in details.items():
+        assert "table lookup" in d[-1], (k, d)
+    want, plain = run(0)
+    for k, d in plain.items():
+        assert "table lookup" not in d[-1], (k, d)
+    for k in got:
+        assert got[k].dtype == want[k].dtype and np.array_equal(got[k].view(np.uint16 if got[k].dtype == np.float16 else np.uint32),
+                                                                  want[k].view(np.uint16 if got[k].dtype == np.float16 else np.uint32)), k
+    with np.errstate(all="ignore"):
+        oa, ob, obias = OTensor(a), OTensor(b), OTensor(bias)
+        ref = (oa.silu() * (ob + obias.broadcast([rows, cols]))).to_numpy()
+        ref2 = (oa * oa.tanh() + ob).to_numpy()
+    for r, g in ((ref, got["silu(a)*(b+bias)"]), (ref2, got["a*tanh(a)+b"])):
+        finite = np.isfinite(r)
+        assert np.array_equal(np.isnan(g), np.isnan(r))
+        assert np.array_equal(g[finite].view(np.uint16), r[finite].view(np.uint16))
 
 
 def test_a_table_lookup_in_place_and_on_a_permuted_tensor(gpu):

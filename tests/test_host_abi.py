@@ -646,6 +646,34 @@ def test_reference_compat_changes_only_the_square_layer_norm(wkf):
     dev.close()
 
 
+def test_a_costly_value_of_one_f16_operand_is_cut_out_as_a_table(wkf):
+    # silu(a) * (b + bias) on f16: silu(a) depends on `a` alone, so from the table threshold on the planner cuts it out of
+    # the fused program, plans a kernel that fills the table (the cut program, marked "!" because its result fed further
+    # arithmetic and keeps the rounding of an interior op) and a map kernel with a `lookup` in its place and the table as
+    # one more argument; below the threshold, with tables off, or on f32 nothing changes
+    dev = wkf.Device.planner()
+    T = wkf.Tensor
+    n = (512, 512)
+
+    def plan(dtype, least):
+        dev.set_map_table(least)
+        a, b = T.new(dev, np.ones(n, dtype=dtype)), T.new(dev, np.ones(n, dtype=dtype))
+        bias = T.new(dev, np.ones((512,), dtype=dtype))
+        t = (a.silu() * (b + bias.broadcast(list(n)))).materialize()
+        return [(k.signature, k.detail) for k in t.kernels()]
+
+    cut = plan(np.float16, 1 << 17)
+    assert len(cut) == 2
+    assert cut[0][0].endswith("load:f16@0;neg:f16(0);exp:f16(1);add_const:f16(2,c0);div:f16(0,3)->4!") and "shape=[65536]" in cut[0][1]
+    assert "lookup:f16(0)" in cut[1][0] and cut[1][0].endswith("|table") and "exp" not in cut[1][0].split("|m0|")[1]
+    assert "table lookup: 65536 values of" in cut[1][1]
+    again = plan(np.float16, 1 << 17)
+    assert len(again) == 1 and again[0][0] == cut[1][0]            # the table is kept per device
+    for other in (plan(np.float16, 1 << 25), plan(np.float16, 0), plan(np.float32, 1 << 17)):
+        assert len(other) == 1 and "lookup" not in other[0][0] and "|table" not in other[0][0]
+    dev.close()
+
+
 def test_a_timer_outlives_its_device_handle(wkf):
     # A timer keeps its device alive like a buffer does (its events go back to that device's pool): destroying the
     # device first and the timer afterwards must find the device still there, and the device goes with the timer.

@@ -29,7 +29,7 @@ bool exact_op(const Program& p, size_t i, MathPolicy policy) {
   if (policy == MathPolicy::Folded) return false;
   for (size_t j = i + 1; j < p.ins.size(); j++)
     if (p.ins[j].a == int(i) || p.ins[j].b == int(i)) return true;  // interior: something reads it
-  return false;
+  return p.result_feeds && int(i) == p.result;                       // ... or something outside the program does
 }
 
 bool has_core(Op o) { return o == Op::Exp || o == Op::Sin || o == Op::Cos; }
@@ -78,7 +78,7 @@ const char* const kRoundH =
 bool is_transcendental(Op o) {
   switch (o) {
     case Op::Load: case Op::AddC: case Op::SubC: case Op::RSubC: case Op::MulC: case Op::DivC: case Op::RDivC: case Op::Sqr:
-    case Op::Neg: case Op::Abs: case Op::Cast: case Op::Add: case Op::Sub: case Op::Mul: case Op::Div: case Op::Sqrt:
+    case Op::Neg: case Op::Abs: case Op::Cast: case Op::Add: case Op::Sub: case Op::Mul: case Op::Div: case Op::Sqrt: case Op::Lookup:
       return false;
     default:
       return true;
@@ -157,6 +157,7 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
     o << "  const " << t << " v" << i << " = ";
     switch (in.op) {
       case Op::Load: o << "x" << in.operand; break;
+      case Op::Lookup: o << "wkf_lookup(" << a << ")"; break;
       case Op::AddC: o << a << " + " << k; break;
       case Op::SubC: o << a << " - " << k; break;
       case Op::RSubC: o << k << " - " << a; break;
@@ -262,6 +263,7 @@ std::string map_signature(const MapSpec& s) {
   for (const auto& i : s.in) o << dtype_name(i.dtype) << (i.linear ? 'L' : 'S') << i.inner_stride << ',';
   o << "|out:" << dtype_name(s.out.dtype) << (s.out.linear ? 'L' : 'S') << s.out.inner_stride;
   o << "|m" << int(s.math) << "|" << s.prog.signature();
+  if (s.table) o << "|table";
   for (size_t j = 0; j < s.more_out.size(); j++)
     o << "|out+:" << dtype_name(s.more_out[j].dtype) << (s.more_out[j].linear ? 'L' : 'S') << s.more_out[j].inner_stride << "|"
       << s.more_prog[j].signature();
@@ -496,7 +498,13 @@ std::string map_source(const MapSpec& s) {
     if (any_round_h) o << kRoundH;
   }
   o << "struct Args { void* p[" << N << "]; u32 nwork; u32 shape[" << R << "]; u32 off[" << N << "]; u32 stride[" << N
-    << "][" << R << "]; float c[" << NC << "]; };\n";
+    << "][" << R << "]; float c[" << NC << "];" << (s.table ? " const unsigned short* table;" : "") << " };\n";
+  // threads per block; a kernel with a table runs 1024 lanes per compute unit around its 128 KiB of LDS
+  const int B = s.table ? kMapTableBlock : kMapBlock;
+  if (s.table)
+    o << "__shared__ __attribute__((aligned(16))) unsigned short wkf_lut[65536];\n"
+         "static __device__ __forceinline__ _Float16 wkf_lookup(_Float16 x) {\n"
+         "  return __builtin_bit_cast(_Float16, wkf_lut[__builtin_bit_cast(unsigned short, x)]);\n}\n";
   std::vector<DType> types;
   for (const auto& i : s.in) types.push_back(i.dtype);
   auto fn = [&](int q) { return q == 0 ? std::string("wkf_expr") : "wkf_expr" + std::to_string(q); };
@@ -525,7 +533,7 @@ std::string map_source(const MapSpec& s) {
   auto is_vec_load = [&](int k) { return V > 1 && (operand(k).linear || operand(k).inner_stride == 1); };
 
   auto emit_index = [&](int j, const char* ind) {
-    o << ind << "const u32 w" << j << " = w_first + " << j * kMapBlock << "u;\n";
+    o << ind << "const u32 w" << j << " = w_first + " << j * B << "u;\n";
     if (need_unravel) {
       o << ind << "u32 rem" << j << " = w" << j << ";\n";
       for (int d = R - 1; d > 0; d--) {
@@ -601,10 +609,22 @@ std::string map_source(const MapSpec& s) {
     for (int j = j0; j < j1; j++) emit_store(j, ind.c_str());
   };
 
-  o << "extern \"C\" __global__ void __launch_bounds__(" << kMapBlock << ") WKF_ENTRY(const Args a) {\n";
-  o << "  const u32 w_block = blockIdx.x * " << kMapBlock * U << "u;\n";
+  o << "extern \"C\" __global__ void __launch_bounds__(" << B << ") WKF_ENTRY(const Args a) {\n";
+  if (s.table) {
+    // the table goes to the LDS once; the block then walks chunks blockIdx.x, blockIdx.x + gridDim.x, ...
+    o << "  typedef u32 wkf_u4 __attribute__((ext_vector_type(4)));\n"
+         "#pragma unroll\n"
+         "  for (int i = 0; i < " << 65536 * 2 / 16 / B << "; i++) ((wkf_u4*)wkf_lut)[threadIdx.x + i * " << B << "u] = ((const wkf_u4*)a.table)[threadIdx.x + i * " << B << "u];\n"
+         "  __syncthreads();\n";
+    o << "  const u32 nchunk = a.nwork / " << B * U << "u + (a.nwork % " << B * U << "u != 0u);\n";
+    o << "  for (u32 chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {\n";
+    o << "  const u32 w_block = chunk * " << B * U << "u;\n";
+  } else {
+    o << "  const u32 w_block = blockIdx.x * " << B * U << "u;\n";
+  }
   o << "  const u32 w_first = w_block + threadIdx.x;\n";
-  o << "  if (w_block + " << kMapBlock * U << "u <= a.nwork) {\n";
+  if (s.table) o << "  if (a.nwork - w_block >= " << B * U << "u) {\n";
+  else o << "  if (w_block + " << B * U << "u <= a.nwork) {\n";
   // Full block: every load is issued before the first use so that U independent
   // 16-byte requests per operand are in flight per lane.
   for (int j = 0; j < U; j++) emit_index(j, "    ");
@@ -617,7 +637,9 @@ std::string map_source(const MapSpec& s) {
     emit_batch(j, j + 1, "        ");
     o << "      }\n    }\n";
   }
-  o << "  }\n}\n";
+  o << "  }\n";
+  if (s.table) o << "  }\n";
+  o << "}\n";
   return o.str();
 }
 
@@ -699,6 +721,10 @@ std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a) {
   nc = std::max<size_t>(1, nc);
   for (size_t i = 0; i < nc; i++) putf(b, i < a.consts.size() ? a.consts[i] : 0.f);
   pad8(b);
+  if (s.table) {
+    if (!a.table) throw Error(WKF_ERR_INVALID_ARG, "map_pack_args: the kernel takes a table");
+    putp(b, const_cast<void*>(a.table));
+  }
   return b;
 }
 

@@ -57,6 +57,9 @@ struct MapSpec {
   std::vector<MapOperandSpec> more_out;
   std::vector<Program> more_prog;
   MathPolicy math = MathPolicy::Stored;
+  // The program holds Op::Lookup instructions: the kernel takes a table of 65536 f16 values as one more argument, copies
+  // it into the LDS of 1024-lane workgroups that stay on their compute unit, and these walk the work items (unroll is 1).
+  bool table = false;
 };
 constexpr int kMaxRank = 6;
 constexpr int kMapBlock = 256;
@@ -83,6 +86,7 @@ struct MapArgs {
   std::vector<uint32_t> offsets;         // per operand, elements
   std::vector<std::vector<uint32_t>> strides;  // per operand, per dim, elements
   std::vector<float> consts;             // of prog, then of every further program
+  const void* table = nullptr;           // MapSpec::table: 65536 f16 values on the device
 };
 std::vector<unsigned char> map_pack_args(const MapSpec& s, const MapArgs& a);
 

@@ -39,6 +39,7 @@ const char* op_name(Op o) {
     case Op::Div: return "div";
     case Op::Pow: return "pow";
     case Op::Load: return "load";
+    case Op::Lookup: return "lookup";
   }
   return "?";
 }
@@ -121,6 +122,7 @@ std::string Program::signature() const {
     }
   }
   s << "->" << result;
+  if (result_feeds) s << "!";
   return s.str();
 }
 

@@ -30,6 +30,7 @@ enum class Op : int {
   Cast = 48,                                                         // to the instruction's dtype
   Add = 64, Sub, Mul, Div, Pow,                                      // pair-wise
   Load = 96,                                                         // read operand #operand
+  Lookup = 97,                                                       // f16 only: the value the kernel's table holds for the bit pattern of `a` (planner-made, never part of a graph)
 };
 inline bool is_const_op(Op o) { return int(o) >= 0 && int(o) <= int(Op::RDivC); }
 inline bool is_unary_op(Op o) { return int(o) >= int(Op::Exp) && int(o) <= int(Op::Neg); }
@@ -134,6 +135,9 @@ struct Program {
   std::vector<Instr> ins;
   std::vector<float> consts;
   int result = -1;
+  // The result is read by further arithmetic outside this program (the program fills a lookup table for a value that
+  // the kernel it was cut from computes in its interior): its last op is evaluated the way an interior op is.
+  bool result_feeds = false;
   DType result_dtype() const { return ins[result].dtype; }
   // Text that identifies the program's structure (constants excluded: they are kernel arguments).
   std::string signature() const;

@@ -320,27 +320,7 @@ void tables_forget(wkf_device* dev) {
 }  // the buffers are released here, outside the lock
 }  // namespace
 
-bool Resolver::try_map_table(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place) {
-  const size_t numel = out.layout.numel();
-  if (st_.fusion != FusionMode::Tree || st_.map_table_min == 0 || numel < std::max<size_t>(st_.map_table_min, 1u << 17) || noalloc_) return false;
-  if (in.size() != 1 || in[0].dtype != DType::F16 || out.dtype != DType::F16 || prog.result_dtype() != DType::F16) return false;
-  // both dense in the same order (any permutation of dimensions, as long as input and output share it), 16-byte aligned
-  if (in[0].layout.strides != out.layout.strides || in[0].layout.offset % 8 || out.layout.offset % 8) return false;
-  {
-    std::vector<std::pair<size_t, size_t>> dims_by_stride;
-    for (size_t d = 0; d < out.layout.shape.size(); d++)
-      if (out.layout.shape[d] != 1) dims_by_stride.push_back({out.layout.strides[d], out.layout.shape[d]});
-    std::sort(dims_by_stride.begin(), dims_by_stride.end());
-    size_t expect = 1;
-    for (const auto& ds : dims_by_stride) {
-      if (ds.first != expect) return false;
-      expect *= ds.second;
-    }
-  }
-  if (numel / 8 > 0xffffffffull || program_cost(prog) < 12 || wkf_device_closing_(dev_)) return false;
-  if ((in[0].layout.offset + numel) * 2 > wkf_buffer_size(in[0].buffer.get()) + 3 || (out.layout.offset + numel) * 2 > wkf_buffer_size(out.buffer.get()) + 3)
-    invalid("map kernel: a layout reaches past the end of its buffer");
-
+BufRef Resolver::map_table_for(const Program& prog) {
   const MathPolicy policy = st_.exact_math ? MathPolicy::Exact : st_.math_f32 ? MathPolicy::Folded : MathPolicy::Stored;
   std::string key = prog.signature() + "|m" + std::to_string(int(policy)) + "|";
   for (float c : prog.consts) {
@@ -385,6 +365,129 @@ bool Resolver::try_map_table(const Program& prog, const std::vector<TensorData>&
     if (mt.tables.size() >= kMaxMapTables) mt.tables.erase(mt.tables.begin());
     mt.tables.push_back({key, table});
   }
+  return table;
+}
+
+BufRef Resolver::cut_table(Program& prog, const std::vector<TensorData>& in, size_t numel, std::string* what) {
+  if (st_.fusion != FusionMode::Tree || st_.map_table_min == 0 || numel < std::max<size_t>(st_.map_table_min, 1u << 17) || noalloc_ ||
+      wkf_device_closing_(dev_))
+    return BufRef();
+  const int n = int(prog.ins.size());
+  // the one operand a value depends on (-1: none yet, -2: several)
+  std::vector<int> leaf(size_t(n), -1);
+  auto join = [](int x, int y) { return x == -1 ? y : y == -1 ? x : x == y ? x : -2; };
+  for (int i = 0; i < n; i++) {
+    const Instr& q = prog.ins[size_t(i)];
+    if (q.op == Op::Lookup) return BufRef();
+    if (q.op == Op::Load) leaf[size_t(i)] = q.operand;
+    else leaf[size_t(i)] = join(q.a >= 0 ? leaf[size_t(q.a)] : -1, q.b >= 0 ? leaf[size_t(q.b)] : -1);
+  }
+  // the instructions a value is computed from, itself included
+  auto cone_of = [&](int f) {
+    std::vector<bool> inc(size_t(n), false);
+    inc[size_t(f)] = true;
+    for (int i = f; i >= 0; i--)
+      if (inc[size_t(i)]) {
+        if (prog.ins[size_t(i)].a >= 0) inc[size_t(prog.ins[size_t(i)].a)] = true;
+        if (prog.ins[size_t(i)].b >= 0) inc[size_t(prog.ins[size_t(i)].b)] = true;
+      }
+    return inc;
+  };
+  // the program that computes value f from its one operand (operand 0 there)
+  auto sub_program = [&](int f) {
+    const std::vector<bool> inc = cone_of(f);
+    Program sub;
+    std::vector<int> id(size_t(n), -1);
+    for (int i = 0; i <= f; i++) {
+      if (!inc[size_t(i)]) continue;
+      Instr q = prog.ins[size_t(i)];
+      if (q.op == Op::Load) q.operand = 0;
+      if (q.a >= 0) q.a = id[size_t(q.a)];
+      if (q.b >= 0) q.b = id[size_t(q.b)];
+      if (q.cslot >= 0) {
+        sub.consts.push_back(prog.consts[size_t(q.cslot)]);
+        q.cslot = int(sub.consts.size()) - 1;
+      }
+      id[size_t(i)] = int(sub.ins.size());
+      sub.ins.push_back(q);
+    }
+    sub.result = id[size_t(f)];
+    sub.result_feeds = f != prog.result;
+    return sub;
+  };
+  int best = -1, best_cost = 0;
+  for (int f = 0; f < n; f++) {
+    const Instr& q = prog.ins[size_t(f)];
+    if (q.op == Op::Load || leaf[size_t(f)] < 0 || q.dtype != DType::F16 || in[size_t(leaf[size_t(f)])].dtype != DType::F16) continue;
+    // (any f16 value of one operand qualifies; the one that takes the most work with it wins, the later of equals: where
+    // other operands come in, where the result is stored, or where a cast leaves f16)
+    const Program sub = sub_program(f);
+    const int cost = program_cost(sub) + (sub.result_feeds && is_unary_op(q.op) ? 7 : 0);
+    if (cost >= best_cost) {
+      best = f;
+      best_cost = cost;
+    }
+  }
+  if (best < 0 || best_cost < 8) return BufRef();   // one interior transcendental is worth the lookup; a few cheap ops are not
+  const Program sub = sub_program(best);
+  BufRef table = map_table_for(sub);
+  // the value becomes a lookup on its operand's load; what only it needed goes away
+  const std::vector<bool> inc = cone_of(best);
+  int load = -1;
+  for (int i = 0; i < best && load < 0; i++)
+    if (inc[size_t(i)] && prog.ins[size_t(i)].op == Op::Load) load = i;
+  Instr lk;
+  lk.op = Op::Lookup;
+  lk.a = load;
+  lk.dtype = DType::F16;
+  prog.ins[size_t(best)] = lk;
+  std::vector<bool> live(size_t(n), false);
+  live[size_t(prog.result)] = true;
+  for (int i = n - 1; i >= 0; i--)
+    if (live[size_t(i)]) {
+      if (prog.ins[size_t(i)].a >= 0) live[size_t(prog.ins[size_t(i)].a)] = true;
+      if (prog.ins[size_t(i)].b >= 0) live[size_t(prog.ins[size_t(i)].b)] = true;
+    }
+  Program cut;
+  cut.consts = prog.consts;   // slots keep their numbers (a slot nothing reads any more costs four bytes of arguments)
+  std::vector<int> id(size_t(n), -1);
+  for (int i = 0; i < n; i++) {
+    if (!live[size_t(i)]) continue;
+    Instr q = prog.ins[size_t(i)];
+    if (q.a >= 0) q.a = id[size_t(q.a)];
+    if (q.b >= 0) q.b = id[size_t(q.b)];
+    id[size_t(i)] = int(cut.ins.size());
+    cut.ins.push_back(q);
+  }
+  cut.result = id[size_t(prog.result)];
+  cut.result_feeds = prog.result_feeds;
+  prog = cut;
+  if (what) *what = sub.signature();
+  return table;
+}
+
+bool Resolver::try_map_table(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place) {
+  const size_t numel = out.layout.numel();
+  if (st_.fusion != FusionMode::Tree || st_.map_table_min == 0 || numel < std::max<size_t>(st_.map_table_min, 1u << 17) || noalloc_) return false;
+  if (in.size() != 1 || in[0].dtype != DType::F16 || out.dtype != DType::F16 || prog.result_dtype() != DType::F16) return false;
+  // both dense in the same order (any permutation of dimensions, as long as input and output share it), 16-byte aligned
+  if (in[0].layout.strides != out.layout.strides || in[0].layout.offset % 8 || out.layout.offset % 8) return false;
+  {
+    std::vector<std::pair<size_t, size_t>> dims_by_stride;
+    for (size_t d = 0; d < out.layout.shape.size(); d++)
+      if (out.layout.shape[d] != 1) dims_by_stride.push_back({out.layout.strides[d], out.layout.shape[d]});
+    std::sort(dims_by_stride.begin(), dims_by_stride.end());
+    size_t expect = 1;
+    for (const auto& ds : dims_by_stride) {
+      if (ds.first != expect) return false;
+      expect *= ds.second;
+    }
+  }
+  if (numel / 8 > 0xffffffffull || program_cost(prog) < 12 || wkf_device_closing_(dev_)) return false;
+  if ((in[0].layout.offset + numel) * 2 > wkf_buffer_size(in[0].buffer.get()) + 3 || (out.layout.offset + numel) * 2 > wkf_buffer_size(out.buffer.get()) + 3)
+    invalid("map kernel: a layout reaches past the end of its buffer");
+
+  BufRef table = map_table_for(prog);
 
   const std::string sig = map_table_signature();
   wkf_kernel* k = kernel(sig, [&] { return map_table_source(); });
@@ -1239,6 +1342,15 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   }
   const size_t nwork = numel / vec;
   spec.unroll = nwork >= (1u << 20) ? st_.map_unroll : nwork >= (1u << 16) ? 2 : 1;
+  // A costly value that depends on one f16 operand only (silu(a) inside silu(a) * (b + bias), the whole chain over a
+  // strided view) is a function of 16 bits: the kernel looks it up in a table held in the LDS instead of computing it.
+  std::string tabled;
+  BufRef table;
+  if (more_out.empty()) table = cut_table(spec.prog, in, numel, &tabled);
+  if (table) {
+    spec.table = true;
+    spec.unroll = 1;
+  }
   size_t bytes = 0;
   std::vector<size_t> cstrides = Layout::contiguous_strides(sp.shape);
   for (size_t k = 0; k < N; k++) {
@@ -1270,6 +1382,7 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   }
   args.consts = prog.consts;
   for (const Program& p : more_prog) args.consts.insert(args.consts.end(), p.consts.begin(), p.consts.end());
+  if (table) args.table = wkf_buffer_ptr(table.get());
 
   std::string sig = map_signature(spec);
   wkf_kernel* k = kernel(sig, [&] { return map_source(spec); });
@@ -1277,12 +1390,19 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   r.kind = "map";
   r.signature = sig;
   r.in_place = in_place;
-  size_t per_block = size_t(kMapBlock) * spec.unroll;
+  size_t per_block = size_t(table ? kMapTableBlock : kMapBlock) * spec.unroll;
   r.grid[0] = to_u32((nwork + per_block - 1) / per_block, "grid");
-  r.block[0] = kMapBlock;
+  r.block[0] = table ? kMapTableBlock : kMapBlock;
+  if (table) {
+    // one workgroup per compute unit keeps the table and walks the chunks
+    wkf_props props;
+    check(wkf_device_props(dev_, &props));
+    r.grid[0] = std::min(r.grid[0], uint32_t(std::max(1, props.compute_units)));
+  }
   std::ostringstream d;
   d << "shape=" << dims(sp.shape) << " vec=" << vec << " unroll=" << spec.unroll << " operands=" << N
     << (in_place ? " in_place" : "");
+  if (table) d << " table lookup: 65536 values of " << tabled;
   if (!more_out.empty()) d << " outputs=" << 1 + more_out.size();
   r.detail = d.str();
   record(std::move(r), k, map_pack_args(spec, args));

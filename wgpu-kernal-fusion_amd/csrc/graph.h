@@ -161,6 +161,11 @@ class Resolver {
   // kernel, over every bit pattern; kept per device, program and constants) and the data is streamed through a
   // lookup in the LDS.  Bit-identical to the ordinary kernel by construction.  False: not applicable, nothing launched.
   bool try_map_table(const Program& prog, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
+  // the table of `prog` (one f16 operand, f16 result) over all 65536 bit patterns, from the device's cache or built now
+  BufRef map_table_for(const Program& prog);
+  // Replaces the costliest value of `prog` that depends on one f16 operand only by a table lookup (Op::Lookup) and returns
+  // the table, or nothing when no value is worth it
+  BufRef cut_table(Program& prog, const std::vector<TensorData>& in, size_t numel, std::string* what);
   void launch_map_tiled(MapSpec& spec, const Space& sp, const std::vector<TensorData>& in, const TensorData& out, bool in_place);
   // `result`: the buffer receives the value of a reduce node (allocation-free mode: the caller's output tensor)
   TensorData alloc(const std::vector<size_t>& shape, DType dt, bool zero, bool result = false);
