@@ -89,6 +89,20 @@ def test_chains_with_interior_transcendentals(gpu, exact):
         assert_ulp(got[i], f(OTensor(x), OTensor(y)).to_numpy(), 1 if exact else 2, f"chain {i}")
 
 
+def test_interior_tanh_on_f32_is_rounded_once(gpu):
+    # a tanh that feeds further arithmetic on f32 has an f64 core of its own (1 - 2 / (exp(2|x|) + 1), a series near zero):
+    # arguments from 1e-30 to beyond saturation, both signs, zeros, infinities and NaN; the product with 1 must be the
+    # correctly rounded tanh (the oracle's float64 tanh rounded to f32; one ulp of slack for the oracle's own libm)
+    rng = np.random.default_rng(11)
+    mags = np.exp(rng.uniform(np.log(1e-30), np.log(30.0), 200000)).astype(np.float32)
+    x = np.concatenate([mags, -mags, np.float32([0.0, -0.0, np.inf, -np.inf, np.nan, 2.0 ** -6, 9.0109, 20.0, 1e30]),
+                        np.linspace(-0.02, 0.02, 4001, dtype=np.float32)])
+    got, want = both(gpu, lambda t: t.tanh() * 1.0, x)
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.signbit(got), np.signbit(want))
+    assert_ulp(got, want, 1, "interior tanh on f32")
+    assert np.mean(got.view(np.uint32) == want.view(np.uint32)) > 0.99999
+
+
 def test_interior_exp_on_f16_is_correctly_rounded_for_every_argument(gpu):
     # an exp that feeds further arithmetic on an f16 tensor goes through the f32 library and, when that cannot
     # decide the f16 rounding, through the f64 core: checked on all 63488 finite f16 values (subnormals included)

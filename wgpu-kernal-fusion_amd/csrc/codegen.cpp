@@ -32,7 +32,7 @@ bool exact_op(const Program& p, size_t i, MathPolicy policy) {
   return p.result_feeds && int(i) == p.result;                       // ... or something outside the program does
 }
 
-bool has_core(Op o) { return o == Op::Exp || o == Op::Sin || o == Op::Cos; }
+bool has_core(Op o) { return o == Op::Exp || o == Op::Sin || o == Op::Cos || o == Op::Tanh; }
 
 // Needs the f64 cores of kernels/math.hip.inc.
 bool uses_math(const Program& p, MathPolicy policy) {
@@ -121,6 +121,7 @@ std::string math_call(Op o, const std::string& a, bool exact, bool far_variant, 
   if (o == Op::Sqrt || !exact) return f + "f(" + a + ")";  // sqrtf is correctly rounded already
   const char* d = wide ? "_d" : "";
   if (o == Op::Exp) return std::string("wkf_exp") + d + "(" + a + ")";
+  if (o == Op::Tanh) return std::string("wkf_tanh") + d + "(" + a + ")";
   if (o == Op::Sin || o == Op::Cos) return "wkf_" + f + (far_variant ? std::string("_far") + d + "(" + a + ")" : std::string(d) + "(" + a + ", far)");
   return (wide ? "" : "(float)") + f + "((double)(" + a + "))";  // the library's f64 routine, rounded once
 }
