@@ -835,6 +835,41 @@ def yardsticks(w, dev, seeded, which, launches):
                               "moved_MiB": moved >> 20, "kernel_us": round(med, 2), "kernel_min_us": round(min(each), 2), "batch_us": round(batch, 2),
                               "GB/s_kernel": round(moved / med * 1e-3), "GB/s_batch": round(moved / batch * 1e-3)})
         out["streams_sized"] = sized
+        # A second pass over what a kernel has just read: the read-only kernel over a piece, then the copy kernel over the
+        # same piece (or over another one, for comparison); the copy's own begin-to-end time, median of 8.  512 MiB are read
+        # elsewhere before every pair so that nothing is left from the pair before.  With ordinary loads in the first pass
+        # the second finds the piece in the 256 MB Infinity Cache; with non-temporal loads it does not.
+        second = []
+        for piece in (64 << 20, 128 << 20):
+            for ntl in (0, 1):
+                ks = {}
+                for mode in (0, 1):
+                    defs = f"#define MODE {mode}\n#define WG 256\n#define U 8\n#define NTL {ntl}\n#define NTS 1\n#define PERSIST 0\n"
+                    ks[mode] = kernel(f"yardstick|stream|{mode}|256|8|{ntl}|1|0", defs + STREAM_SRC, "wkf_stream")
+
+                def go(k, nbytes, off_s, off_d, timer=None):
+                    n4 = nbytes // 16
+                    g, b = (c_uint32 * 3)(n4 // (256 * 8), 1, 1), (c_uint32 * 3)(256, 1, 1)
+                    a = struct.pack("PPQP", lib.wkf_buffer_ptr(src_b) + off_s, lib.wkf_buffer_ptr(dst_b) + off_d, n4, lib.wkf_buffer_ptr(src2_b))
+                    assert lib.wkf_launch(dev._h, k, g, b, 0, a, len(a), timer) == 0
+
+                times = {"same": [], "other": []}
+                for it in range(10):
+                    for which in ("same", "other"):
+                        go(ks[1], 512 << 20, 512 << 20, 0)
+                        go(ks[1], piece, 0, 0)
+                        t = c_void_p()
+                        assert lib.wkf_timer_create(dev._h, byref(t)) == 0
+                        go(ks[0], piece, 0 if which == "same" else (256 << 20), 0, t)
+                        dev.sync()
+                        ns = ctypes.c_uint64()
+                        assert lib.wkf_timer_elapsed_ns(t, byref(ns)) == 0
+                        lib.wkf_timer_destroy(t)
+                        times[which].append(ns.value / 1e3)
+                second.append({"what": f"copy of {piece >> 20} MiB after a read-only pass with {'non-temporal' if ntl else 'ordinary'} loads",
+                               "after_reading_the_same_piece_us": round(float(np.median(times["same"][2:])), 2),
+                               "after_reading_another_piece_us": round(float(np.median(times["other"][2:])), 2)})
+        out["second_pass"] = second
         for name in ("copy", "read-only", "write-only", "two reads + one write"):
             best = max((r for r in rows if r["what"].startswith(name)), key=lambda r: r["GB/s"])
             out["best_" + name.replace("-", "_").replace(" + ", "_").replace(" ", "_")] = best
