@@ -113,6 +113,10 @@ def test_interior_exp_on_f16_is_correctly_rounded_for_every_argument(gpu):
     assert_ulp(got, want, 0, "exp on f16")
     got, want = both(gpu, lambda t: t / (1.0 + (-t).exp()), x)  # silu, as the composite builds it
     assert_ulp(got, want, 0, "silu on f16")
+    with np.errstate(all="ignore"):
+        got, want = both(gpu, lambda t: t.sqrt() * 1.0, x)      # a root that feeds further arithmetic (negative arguments: NaN)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert_ulp(got[~np.isnan(want)], want[~np.isnan(want)], 0, "interior sqrt on f16")
 
 
 @pytest.mark.parametrize("op", sorted(TRANS_UNARY), ids=str)
@@ -1245,6 +1249,69 @@ def test_a_costly_value_of_one_f16_operand_inside_a_larger_map_is_looked_up(gpu)
         finite = np.isfinite(r)
         assert np.array_equal(np.isnan(g), np.isnan(r))
         assert np.array_equal(g[finite].view(np.uint16), r[finite].view(np.uint16))
+
+
+def test_random_f16_maps_agree_with_and_without_tables(gpu):
+    # Random fused maps over three f16 operands (unary, literal, pair-wise ops, casts to f32 and back, values used more
+    # than once): whatever value the planner cuts out into a table, the kernel must give the bits of the ordinary kernel.
+    rows, cols = 300, 520
+    rng0 = np.random.default_rng(900)
+    hosts = [data((rows, cols), -4, 4, np.float16, 901 + i) for i in range(3)]
+    hosts[0].reshape(-1)[:65536] = np.arange(65536, dtype=np.uint16).view(np.float16)
+    hosts[1].reshape(-1)[:65536] = rng0.permutation(65536).astype(np.uint16).view(np.float16)
+    unary = ["exp", "sin", "cos", "tanh", "abs", "sqrt", "log", "atan", "sinh", "sqr"]
+    api = HipAPI(gpu)
+
+    def build(seed, leaves):
+        rng = np.random.default_rng(seed)
+        vals = list(leaves)           # (tensor, is_f16)
+        for _ in range(int(rng.integers(4, 10))):
+            kind = rng.integers(0, 10)
+            t, h = vals[int(rng.integers(0, len(vals)))]
+            if kind < 4:
+                nv = (getattr(t, unary[int(rng.integers(0, len(unary)))])(), h)
+            elif kind < 6:
+                c = float(np.float16(rng.uniform(-2, 2)))
+                nv = ([t + c, t * c, c - t, t / (abs(c) + 0.5)][int(rng.integers(0, 4))], h)
+            elif kind < 9:
+                same = [v for v in vals if v[1] == h]
+                u = same[int(rng.integers(0, len(same)))][0]
+                nv = ([t + u, t - u, t * u, t / u][int(rng.integers(0, 4))], h)
+            else:
+                nv = (t.cast(0 if h else 1), not h)
+            vals.append(nv)
+        # the result joins the last value with one of each other operand's, so that several operands come in
+        out, h = vals[-1]
+        for leaf, lh in leaves[1:]:
+            out = out + (leaf if h == lh else leaf.cast(1 if h else 0))
+        return out
+
+    def run(least, seeds):
+        gpu.set_map_table(least)
+        try:
+            outs, tabled = [], 0
+            for seed in seeds:
+                t = build(seed, [(api.tensor(hh), True) for hh in hosts])
+                if gpu.is_planner:
+                    t.materialize()
+                    continue
+                outs.append(hip_values(t))
+                tabled += any("table lookup" in k.detail for k in t.kernels())
+            return outs, tabled
+        finally:
+            gpu.set_map_table(1 << 25)
+
+    seeds = range(40)
+    if gpu.is_planner:
+        run(1 << 17, seeds)
+        run(0, seeds)
+        hip_values(api.tensor(hosts[0]) * 2.0)
+    got, tabled = run(1 << 17, seeds)
+    want, none = run(0, seeds)
+    for seed, (g, w_) in enumerate(zip(got, want)):
+        bits = np.uint16 if g.dtype == np.float16 else np.uint32
+        assert g.dtype == w_.dtype and np.array_equal(g.view(bits), w_.view(bits)), seed
+    assert none == 0 and tabled >= 12, (tabled, none)   # about half of these graphs hold a value worth a table
 
 
 def test_a_table_lookup_in_place_and_on_a_permuted_tensor(gpu):

@@ -646,6 +646,22 @@ def test_reference_compat_changes_only_the_square_layer_norm(wkf):
     dev.close()
 
 
+@pytest.mark.parametrize("dtype", [np.float16, np.float32], ids=["f16", "f32"])
+def test_every_unary_op_compiles_where_its_value_feeds_further_work(wkf, dtype):
+    # the generator picks a different evaluation for an op whose value is read again (f64 cores, f16 roundings decided in
+    # f32, ...): every unary op, followed by a literal op, inside a reduction's chain and in front of a cast, must give a
+    # kernel that compiles (an interior sqrt on f16 once named a helper its kernel did not include)
+    dev = wkf.Device.planner()
+    x = wkf.Tensor.new(dev, np.ones((64, 64), dtype=dtype))
+    ops = ["exp", "exp2", "log", "log2", "sqr", "sqrt", "sin", "cos", "tan", "asin", "acos", "atan", "sinh", "cosh", "tanh",
+           "asinh", "acosh", "atanh", "abs"]
+    for op in ops:
+        for graph in (getattr(x, op)() * 2.0, getattr(x, op)().sum(1), getattr(x, op)().cast(wkf.F32 if dtype == np.float16 else wkf.F16) + 1.0):
+            graph.materialize()
+            assert len(graph.kernels()) == 1, op
+    dev.close()
+
+
 def test_a_costly_value_of_one_f16_operand_is_cut_out_as_a_table(wkf):
     # silu(a) * (b + bias) on f16: silu(a) depends on `a` alone, so from the table threshold on the planner cuts it out of
     # the fused program, plans a kernel that fills the table (the cut program, marked "!" because its result fed further

@@ -209,7 +209,9 @@ void emit_program_variant(std::ostringstream& o, const Program& p, const std::st
           break;
         }
         std::string call = math_call(in.op, h ? "(float)" + a : a, exact, far_variant, h);
-        if (h && exact) o << "wkf_round_h(" << call << ")";
+        // (sqrtf of an f16 value is the correctly rounded f32 root, and 24 bits are enough for the second rounding to f16
+        // to be harmless: no f64 step, whatever reads the value)
+        if (h && exact && in.op != Op::Sqrt) o << "wkf_round_h(" << call << ")";
         else o << (h ? "(_Float16)" : "") << call;
       }
     }
