@@ -89,11 +89,12 @@ def measure_kernels(dev, wl, steps, warmup):
         wl.step(i)
     dev.sync()
     samples, kinds, details = [], None, None
-    # The next step is enqueued before the times of the step before it are read (a different input variant, so its
-    # kernel records are not the ones being read): reading a time waits for its kernel, and on some machines a GPU that
-    # waits for the host between two short kernels drops its clocks (seen: 30 us per launch read one by one against
-    # 23 us for a 128 MiB map kernel).  With a single variant the steps are read one by one.
-    ahead = len(wl.variants) >= 2
+    # Steps are enqueued ahead of the step whose times are read (other input variants, so their kernel records are
+    # not the ones being read), as many as there are variants to spare: reading a time waits for its kernel, and on some
+    # machines a GPU that waits for the host between two short kernels drops its clocks (seen: 28-30 us per launch read
+    # one by one against 23 us for a 128 MiB map kernel whose vector ALUs are busy 60 % of the time).  With a single
+    # variant the steps are read one by one.
+    depth = len(wl.variants) - 1
 
     def read(outs):
         nonlocal kinds, details
@@ -104,17 +105,13 @@ def measure_kernels(dev, wl, steps, warmup):
         kinds = [k.kind for k in ks]
         details = [k.detail for k in ks]
 
-    before = None
+    pending = []
     for i in range(steps):
-        outs = wl.step(i)
-        if not ahead:
-            read(outs)
-            continue
-        if before is not None:
-            read(before)
-        before = outs
-    if before is not None:
-        read(before)
+        pending.append(wl.step(i))
+        if len(pending) > depth:
+            read(pending.pop(0))
+    for outs in pending:
+        read(outs)
     arr = np.array(samples, dtype=np.float64) / 1e3  # [step][kernel] in us
     med, mn = np.median(arr, axis=0), arr.min(axis=0)
     total = arr.sum(axis=1)
@@ -1006,7 +1003,9 @@ def main():
                     continue
                 settle(dev, one)  # the CPU port and the uploads before this row left the GPU idle
                 measured = measure_kernels(dev, one, steps, warm)
+                settle(dev, one, 0.1)  # reading the per-launch times above left the GPU waiting for the host
                 wall_s = measure_wall(dev, one, steps, 5)
+                settle(dev, one, 0.1)
                 batch_us = round(measure_batch(w, dev, one, steps, 5), 2)
                 row = summarise(one, measured, wall_s, steps, batch_us)
                 row["key"] = key
