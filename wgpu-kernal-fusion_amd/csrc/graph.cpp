@@ -1367,6 +1367,8 @@ void Resolver::launch_map(const Program& prog, const std::vector<TensorData>& in
   spec.nontemporal = bytes >= st_.nontemporal_bytes;
 
   MapArgs args;
+  // (a block computes the index of its first work item plus up to 16384: that sum stays below 2^32 as well)
+  if (nwork > 0xffffffffull - (size_t(1) << 16)) throw Error(WKF_ERR_UNSUPPORTED, "map kernel: more than 2^32 - 2^16 work items");
   args.nwork = to_u32(nwork, "tensor size");
   for (size_t d = 0; d < R; d++) args.shape.push_back(to_u32(d == R - 1 ? sp.shape[d] / vec : sp.shape[d], "shape"));
   for (size_t k = 0; k < N; k++) {
