@@ -259,6 +259,39 @@ def test_transposed_operands_with_aligned_shapes(gpu, dtype):
         assert np.array_equal(alone[i], g), i
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float16], ids=["f32", "f16"])
+def test_large_transposed_operands_take_tiles_of_128(gpu, dtype):
+    # with four-element accesses, both extents beyond 128, tiles enough for the chip twice over and room in the LDS for two
+    # workgroups per compute unit, the tile is 128 x 128: ragged edges on both sides (3004 = 23 x 128 + 60, 2956 = 23 x 128
+    # + 12), a straight second operand, a per-row scalar, a batch in front; two crossed f32 inputs keep 64 x 64 tiles
+    api = HipAPI(gpu)
+    a = data((3004, 2956), -2, 2, dtype, 31)
+    b = data((2956, 3004), -2, 2, dtype, 32)
+    c = data((6, 1028, 1156), -2, 2, dtype, 33)
+    r = data((2956,), 0.5, 2, dtype, 34)
+
+    def progs(ta, tb, tc, tr):
+        return [ta.transpose(0, 1) + 1.0,
+                ta.transpose(0, 1) * tb - tb,
+                (ta.transpose(0, 1) + tb) / tr.broadcast([3004, 2956]).transpose(0, 1),
+                tc.transpose(1, 2) * 2.0,
+                ta.transpose(0, 1) * tb.transpose(0, 1).transpose(0, 1) + ta.slice([(4, 3004), (0, 2952)]).transpose(0, 1).resize([2956, 3004])]
+
+    ts = progs(api.tensor(a), api.tensor(b), api.tensor(c), api.tensor(r))
+    got = [hip_values(t) for t in ts]
+    for i, t in enumerate(ts[:4]):
+        assert any(k.kind == "map" and "tiled" in k.detail and "tile=128" in k.detail for k in t.kernels()), (i, [k.detail for k in t.kernels()])
+    want = progs(OTensor(a), OTensor(b), OTensor(c), OTensor(r))
+    for i, (g, w) in enumerate(zip(got, want)):
+        assert_ulp(g, w.to_numpy(), 0, f"program {i}")
+    # two crossed f32 inputs: their tiles of 128 would leave one workgroup per compute unit
+    two = api.tensor(a).transpose(0, 1) * api.tensor(np.ascontiguousarray(b.T)).transpose(0, 1)
+    g2 = hip_values(two)
+    assert any("tiled" in k.detail for k in two.kernels())
+    assert ("tile=128" in " ".join(k.detail for k in two.kernels())) == (dtype == np.float16)
+    assert_ulp(g2, (OTensor(a).transpose(0, 1) * OTensor(np.ascontiguousarray(b.T)).transpose(0, 1)).to_numpy(), 0, "two crossed inputs")
+
+
 def test_same_results_under_both_fusion_modes(gpu):
     a, b = data((64, 96), -2, 2, np.float32, 11), data((64, 96), 0.5, 2, np.float32, 12)
     api = HipAPI(gpu)

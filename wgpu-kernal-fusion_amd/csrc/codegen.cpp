@@ -274,6 +274,7 @@ std::string map_signature(const MapSpec& s) {
     o << "|tile" << s.tile_dim << ':';
     for (size_t k = 0; k < s.in.size(); k++) o << (s.crossed[k] ? 'x' : '-');
     if (s.tile_vec > 1) o << "|tv" << s.tile_vec;
+    if (s.tile_size != 64) o << "|ts" << s.tile_size;
   }
   return o.str();
 }
@@ -288,6 +289,8 @@ std::string map_tiled_vec_source(const MapSpec& s) {
   const int N = int(s.in.size()) + 1;
   const int R = s.rank, TA = s.tile_dim, TB = s.rank - 1;
   const int NC = s.prog.consts.empty() ? 1 : int(s.prog.consts.size());
+  // T x T tile; LQ lanes of four elements cover a tile row, the block's 256 lanes RP rows a pass, NP passes the tile
+  const int T = s.tile_size, LQ = T / 4, RP = kMapBlock / LQ, NP = T / RP;
   std::ostringstream o;
   o << kPrelude;
   if (uses_math(s.prog, s.math)) o << kMath;
@@ -305,17 +308,17 @@ std::string map_tiled_vec_source(const MapSpec& s) {
   o << "extern \"C\" __global__ void __launch_bounds__(" << kMapBlock << ") WKF_ENTRY(const Args a) {\n";
   for (int k = 0; k < N - 1; k++)
     if (s.crossed[k])
-      o << "  __shared__ " << ctype(dt(k)) << " tile" << k << "[" << kMapTile << "][" << kMapTile + (dtype_size(dt(k)) == 2 ? 2 : 1) << "];\n";
-  o << "  const u32 q = threadIdx.x & 15u, r = threadIdx.x >> 4;\n";
+      o << "  __shared__ " << ctype(dt(k)) << " tile" << k << "[" << T << "][" << T + (dtype_size(dt(k)) == 2 ? 2 : 1) << "];\n";
+  o << "  const u32 q = threadIdx.x & " << LQ - 1 << "u, r = threadIdx.x / " << LQ << "u;\n";
   o << "  const u32 A = a.shape[" << TA << "], B = a.shape[" << TB << "];\n";
-  o << "  const u32 tiles_a = (A + 63u) / 64u, tiles_b = (B + 63u) / 64u;\n";
+  o << "  const u32 tiles_a = (A + " << T - 1 << "u) / " << T << "u, tiles_b = (B + " << T - 1 << "u) / " << T << "u;\n";
   // Tiles are walked along b, each row of tiles starting one tile further on (a diagonal order): workgroups that run
   // at the same time then touch rows of the crossed operands whose distance is not a fixed multiple of 64 rows
   // (measured on an f32 [8192,8192] transposing copy: 3959 -> 4582 GB/s, with the non-temporal bits 5082).
   o << "  u32 rem = blockIdx.x;\n";
   o << "  const u32 tb_ = rem % tiles_b; rem /= tiles_b;\n";
   o << "  const u32 ta_ = rem % tiles_a; rem /= tiles_a;\n";
-  o << "  const u32 b0 = ((tb_ + ta_) % tiles_b) * 64u, a0 = ta_ * 64u;\n";
+  o << "  const u32 b0 = ((tb_ + ta_) % tiles_b) * " << T << "u, a0 = ta_ * " << T << "u;\n";
   std::vector<int> others;
   for (int d = R - 2; d >= 0; d--)
     if (d != TA) others.push_back(d);
@@ -334,22 +337,22 @@ std::string map_tiled_vec_source(const MapSpec& s) {
   for (int k = 0; k < N - 1; k++) {
     if (!s.crossed[k]) continue;
     std::string vt = vtype(dt(k), 4);
-    o << "  {\n    " << vt << " v[4];\n";
+    o << "  {\n    " << vt << " v[" << NP << "];\n";
     o << "    const u32 aa = min(a0 + q * 4u, A - 4u);\n";
-    o << "#pragma unroll\n    for (int j = 0; j < 4; j++) {\n";
-    o << "      const u32 bb = min(b0 + r + 16u * j, B - 1u);\n";
+    o << "#pragma unroll\n    for (int j = 0; j < " << NP << "; j++) {\n";
+    o << "      const u32 bb = min(b0 + r + " << RP << "u * j, B - 1u);\n";
     o << "      v[j] = " << (s.nontemporal ? "__builtin_nontemporal_load(" : "*(") << "(const " << vt << "*)(" << ptr(k) << " + (base" << k
       << " + aa + bb * a.stride[" << k << "][" << TB << "])));\n    }\n";
-    o << "#pragma unroll\n    for (int j = 0; j < 4; j++)\n#pragma unroll\n      for (int e = 0; e < 4; e++) tile" << k
-      << "[r + 16u * j][q * 4u + e] = v[j][e];\n  }\n";
+    o << "#pragma unroll\n    for (int j = 0; j < " << NP << "; j++)\n#pragma unroll\n      for (int e = 0; e < 4; e++) tile" << k
+      << "[r + " << RP << "u * j][q * 4u + e] = v[j][e];\n  }\n";
   }
   o << "  __syncthreads();\n";
   // phase 2: a vector along the last dim per lane
   o << "  const u32 bb = min(b0 + q * 4u, B - 4u);\n";
   o << "  const bool b_live = b0 + q * 4u < B;\n";
   std::string ovt = vtype(s.out.dtype, 4);
-  o << "#pragma unroll\n  for (int j = 0; j < 4; j++) {\n";
-  o << "    const u32 al = r + 16u * j, aa = a0 + al, ac = min(aa, A - 1u);\n";
+  o << "#pragma unroll\n  for (int j = 0; j < " << NP << "; j++) {\n";
+  o << "    const u32 al = r + " << RP << "u * j, aa = a0 + al, ac = min(aa, A - 1u);\n";
   for (int k = 0; k < N - 1; k++) {
     if (s.crossed[k]) continue;
     if (s.in[k].inner_stride == 1)

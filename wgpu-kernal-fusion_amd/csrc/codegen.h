@@ -44,6 +44,9 @@ struct MapSpec {
   // tile extents are multiples of 4, every other stride and every offset too); non-crossed inputs then have
   // inner_stride 1 (a vector per lane) or 0 (one value per tile row)
   int tile_vec = 1;
+  // edge of the square tile: 64, or 128 with tile_vec == 4 when the operands are large and the tiles of the crossed
+  // inputs leave room for two workgroups per compute unit (longer runs of consecutive bytes per row of a tile)
+  int tile_size = 64;
   std::vector<bool> crossed;         // per input; used when tile_dim >= 0
   int rank;                          // rank of the coalesced iteration space (1..kMaxRank)
   int vec;                           // elements per work item: 1, 2, 4 or 8

@@ -34,6 +34,7 @@ struct Settings {
   int map_unroll = 4;             // work items per thread in large map kernels (WKF_MAP_UNROLL overrides: 1, 2, 4, 8)
   bool reference_compat = false;  // composites keep the reference's text where it differs in value from what it means: layer_norm's weight through Tensor::broadcast (indexed by row on square inputs)
   bool exact_math = false;        // every transcendental through an f64 core (MathPolicy::Exact)
+  bool map_tile_128 = true;       // transposing map kernels may take 128 x 128 tiles (WKF_MAP_TILE_128=0: always 64 x 64)
   bool math_f32 = false;          // measurement only (WKF_MATH_F32=1): map kernels take the f32 library for every transcendental, outside the 2-ulp bound of fused chains; shows what the f64 cores cost
   size_t nontemporal_bytes = size_t(32) << 20;  // map kernels moving at least this much use streaming loads/stores
   int reduce_threads = 0;         // lanes per row in row reduces; 0 = chosen from the shape (WKF_REDUCE_THREADS overrides)

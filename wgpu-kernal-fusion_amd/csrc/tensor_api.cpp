@@ -122,6 +122,7 @@ Settings settings_for(wkf_device* dev) {
     if (const char* u = getenv("WKF_GEMM_DMA")) st.gemm_dma = atoi(u) != 0;
     if (const char* u = getenv("WKF_GEMM_FLEX")) st.gemm_flex = !(u[0] == '0' && u[1] == 0);
     if (const char* u = getenv("WKF_MATH_F32")) st.math_f32 = atoi(u) != 0;
+    if (const char* u = getenv("WKF_MAP_TILE_128")) st.map_tile_128 = atoi(u) != 0;
     if (const char* u = getenv("WKF_MAP_TABLE_MIN")) st.map_table_min = size_t(std::max(0ll, atoll(u)));
     if (const char* u = getenv("WKF_ROW_SPLIT")) st.row_split = atoi(u) != 0;
     if (const char* u = getenv("WKF_ROW_TEAM")) st.row_team = atoi(u) != 0;
