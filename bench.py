@@ -70,9 +70,12 @@ class Workload:
         self.joint = joint  # the package's materialize_many: the tensors of a step are materialised in ONE pass
         self.cpu = cpu
 
-    def step(self, i):
-        """Launches step i; returns the tensors whose kernel records describe it."""
+    def step(self, i, fresh=False):
+        """Launches step i; returns the tensors whose kernel records describe it.  `fresh`: through new handles on the same
+        graph nodes, so that the records of earlier steps stay readable while later ones are already enqueued."""
         ts = self.variants[i % len(self.variants)]
+        if fresh:
+            ts = [t.clone() for t in ts]
         if self.joint:
             self.joint(ts)
             return ts[:1]
@@ -89,12 +92,11 @@ def measure_kernels(dev, wl, steps, warmup):
         wl.step(i)
     dev.sync()
     samples, kinds, details = [], None, None
-    # Steps are enqueued ahead of the step whose times are read (other input variants, so their kernel records are
-    # not the ones being read), as many as there are variants to spare: reading a time waits for its kernel, and on some
+    # Sixteen steps are enqueued ahead of the step whose times are read, each through handles of its own (its kernel
+    # records stay readable, its result lives until it has been read): reading a time waits for its kernel, and on some
     # machines a GPU that waits for the host between two short kernels drops its clocks (seen: 28-30 us per launch read
-    # one by one against 23 us for a 128 MiB map kernel whose vector ALUs are busy 60 % of the time).  With a single
-    # variant the steps are read one by one.
-    depth = len(wl.variants) - 1
+    # one by one against 23 us for a 128 MiB map kernel whose vector ALUs are busy 60 % of the time).
+    depth = 16
 
     def read(outs):
         nonlocal kinds, details
@@ -107,11 +109,11 @@ def measure_kernels(dev, wl, steps, warmup):
 
     pending = []
     for i in range(steps):
-        pending.append(wl.step(i))
+        pending.append(wl.step(i, fresh=True))
         if len(pending) > depth:
             read(pending.pop(0))
-    for outs in pending:
-        read(outs)
+    while pending:
+        read(pending.pop(0))
     arr = np.array(samples, dtype=np.float64) / 1e3  # [step][kernel] in us
     med, mn = np.median(arr, axis=0), arr.min(axis=0)
     total = arr.sum(axis=1)
