@@ -160,6 +160,36 @@ class Tensor {
     for (float f : values) v.push_back(D::from_float(f));
     return Tensor(dev, shape, v);
   }
+  // The nested-array forms of `IntoTensor` (src/tensor.rs:646-760): `Tensor::new(&device, &[[1., 2.], [3., 4.]])` is
+  // `Tensor<2>::from(dev, {{1, 2}, {3, 4}})`; every row (and every matrix of a rank-3 literal) must have the same length.
+  static Tensor from(const Device& dev, std::initializer_list<float> v) {
+    static_assert(R == 1, "a flat list is a rank-1 tensor");
+    return from_floats(dev, {v.size()}, v);
+  }
+  static Tensor from(const Device& dev, std::initializer_list<std::initializer_list<float>> rows) {
+    static_assert(R == 2, "a list of lists is a rank-2 tensor");
+    const size_t cols = rows.size() ? rows.begin()->size() : 0;
+    std::vector<element> flat;
+    for (const auto& r : rows) {
+      if (r.size() != cols) throw Error(WKF_ERR_INVALID_ARG, "Tensor::from: rows of different lengths");
+      for (float f : r) flat.push_back(D::from_float(f));
+    }
+    return Tensor(dev, {rows.size(), cols}, flat);
+  }
+  static Tensor from(const Device& dev, std::initializer_list<std::initializer_list<std::initializer_list<float>>> mats) {
+    static_assert(R == 3, "a list of lists of lists is a rank-3 tensor");
+    const size_t rows = mats.size() ? mats.begin()->size() : 0;
+    const size_t cols = rows ? mats.begin()->begin()->size() : 0;
+    std::vector<element> flat;
+    for (const auto& m : mats) {
+      if (m.size() != rows) throw Error(WKF_ERR_INVALID_ARG, "Tensor::from: matrices of different heights");
+      for (const auto& r : m) {
+        if (r.size() != cols) throw Error(WKF_ERR_INVALID_ARG, "Tensor::from: rows of different lengths");
+        for (float f : r) flat.push_back(D::from_float(f));
+      }
+    }
+    return Tensor(dev, {mats.size(), rows, cols}, flat);
+  }
   // arange / arange_step, src/composite/arange.rs:4-12 (rank 1)
   static Tensor arange(const Device& dev, float start, float end, float step = 1.0f) {
     static_assert(R == 1, "arange builds a rank-1 tensor");

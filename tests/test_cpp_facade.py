@@ -72,6 +72,18 @@ PROGRAM = textwrap.dedent(r"""
         expect(Half::from_float(65520.0f).bits == 0x7c00 && Half::from_float(65519.0f).bits == 0x7bff, "overflow boundary");
         expect(Half::from_float(0x1p-25f).bits == 0 && Half::from_float(0x1.000002p-25f).bits == 1, "underflow boundary");
 
+        // the nested-literal constructors build the same tensors as shape + flat data
+        {
+          auto n2 = Tensor<2, F32>::from(dev, {{1, 2}, {3, 4}, {5, 6}});
+          auto n3 = Tensor<3, F16>::from(dev, {{{1, 2, 3}}, {{4, 5, 6}}});
+          auto n1 = Tensor<1, F32>::from(dev, {7, 8, 9});
+          expect(n2.shape()[0] == 3 && n2.shape()[1] == 2 && n3.shape()[0] == 2 && n3.shape()[1] == 1 && n3.shape()[2] == 3 && n1.shape()[0] == 3, "nested literals: shapes");
+          expect(n2.as_slice()[{2, 0}] == 5.0f && n3.as_slice()[{1, 0, 2}] == 6.0f && n1.as_slice()[{1}] == 8.0f, "nested literals: values");
+          bool ragged = false;
+          try { Tensor<2, F32>::from(dev, {{1, 2}, {3}}); } catch (const wkf::Error& e) { ragged = e.code == WKF_ERR_INVALID_ARG; }
+          expect(ragged, "ragged literal throws");
+        }
+
         // shapes travel with the graph
         auto s = ((x * 2.0f) + 1.0f).sum(1);
         expect(s.shape()[0] == 3, "shape of a reduce");
