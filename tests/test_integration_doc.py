@@ -1,4 +1,4 @@
-"""INTEGRATION.md shows the `extern "C"` block a maintainer of the reference crate would add.  No Rust toolchain
+"""The integration guide at the repository root shows the `extern "C"` block a maintainer of the reference crate would add.  No Rust toolchain
 exists here to compile it, so this test keeps it mechanically in step with the headers: every function it declares
 exists in include/*.h with the same number of arguments and matching argument and return types, and every
 function of include/wkf_tensor.h (the level the block says it covers) is declared in it."""
@@ -6,6 +6,7 @@ import os
 import re
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GUIDE = "INTEGRATION.md"
 
 
 def _strip_c(text):
@@ -52,7 +53,7 @@ def _rust_type(t):
 
 
 def _rust_functions():
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    text = open(os.path.join(ROOT, GUIDE)).read()
     block = text[text.index('extern "C" {'):]
     block = block[:block.index("\n}\n")]
     block = re.sub(r"//[^\n]*", " ", block)
@@ -68,9 +69,9 @@ def test_extern_block_matches_the_headers():
     c, rust = _c_functions(), _rust_functions()
     assert len(rust) >= 50
     for name, (ret, params) in rust.items():
-        assert name in c, f"INTEGRATION.md declares {name}, which no header declares"
+        assert name in c, f"the integration guide declares {name}, which no header declares"
         header, cret, cparams = c[name]
-        assert len(params) == len(cparams), f"{name}: {len(params)} arguments in INTEGRATION.md, {len(cparams)} in {header}"
+        assert len(params) == len(cparams), f"{name}: {len(params)} arguments in the integration guide, {len(cparams)} in {header}"
         for i, (rp, cp) in enumerate(zip(params, cparams)):
             cp_type = re.sub(r"\b\w+\s*$", "", cp) if re.search(r"[\s*]\w+\s*$", cp) else cp   # drop the parameter's name
             assert _rust_type(rp) == _c_type(cp_type), f"{name}, argument {i}: `{rp.strip()}` against `{cp}`"
@@ -83,4 +84,4 @@ def test_extern_block_matches_the_headers():
 def test_extern_block_covers_the_tensor_level():
     c, rust = _c_functions(), _rust_functions()
     missing = sorted(n for n, (header, _, _) in c.items() if header == "wkf_tensor.h" and n not in rust)
-    assert not missing, f"include/wkf_tensor.h declares these, INTEGRATION.md does not: {missing}"
+    assert not missing, f"include/wkf_tensor.h declares these, the integration guide does not: {missing}"
